@@ -1,0 +1,185 @@
+/*
+ * llmk.h — C ABI of the MI355X (gfx950) kernel library behind llm.c's GPT-2 training step.
+ *
+ * One entry point per kernel launcher of the reference (karpathy/llm.c, llmc/ *.cuh), same
+ * argument order and meaning, with
+ *     floatX*       -> void*   (bf16 in libllmk_bf16.so, fp32 in libllmk_fp32.so; the
+ *                               precision is a property of the shared object, as PRECISION=
+ *                               is of the reference build, reference Makefile:232-244)
+ *     cudaStream_t  -> void*   (a hipStream_t; NULL = the default stream)
+ *     templates / std::bool_constant / default arguments -> plain int / explicit arguments.
+ * Citations give the reference launcher each function replaces (paths relative to the
+ * reference checkout).
+ *
+ * Contract (same as the reference's launchers):
+ *   - the caller owns every buffer; functions enqueue work on `stream` and return without
+ *     waiting (exception: llmk_encoder_backward builds its buckets on the host first);
+ *   - a single host thread drives the library;
+ *   - no entry point here allocates device memory per call. GEMMs whose output is smaller than
+ *     the machine (weight gradients) split the contraction and use one library-owned
+ *     workspace that grows to the largest request seen and is then reused (the role of the
+ *     reference's cublaslt_workspace, llmc/cublas_common.h:28-31);
+ *   - errors: a failed HIP call or a violated shape precondition prints a message and exits
+ *     (llmc/cuda_common.h:52-58). llmk_set_error_mode(1) makes the library record the
+ *     message and return instead, for tests; read it with llmk_last_error().
+ *
+ * Shape preconditions: C % 8 == 0 (bf16) / C % 4 == 0 (fp32) for every row length,
+ * head size 64 for attention (C == 64 * NH), 16-byte aligned pointers.
+ */
+#ifndef LLMK_H
+#define LLMK_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* ---- library / device ------------------------------------------------------------------ */
+
+/* Selects the device and reads its properties (reference: common_start, train_gpt2.cu:1173-1200). */
+void llmk_init(int device);
+void llmk_shutdown(void);
+/* "bf16" or "fp32": the floatX of this shared object (reference: PRECISION_MODE, llmc/cuda_common.h:68-92) */
+const char* llmk_precision(void);
+/* sizeof(floatX) */
+int llmk_sizeof_floatx(void);
+/* multiProcessorCount / maxThreadsPerMultiProcessor / name of cudaDeviceProp (llmc/cuda_common.h:27) */
+void llmk_device_props(int* num_cu, int* max_threads_per_cu, char* name256);
+void llmk_set_error_mode(int record_instead_of_exit);
+const char* llmk_last_error(void); /* "" when none; cleared by llmk_clear_error */
+void llmk_clear_error(void);
+
+/* Per-kernel timing (no launcher counterpart in the reference, which marks the same places with NVTX
+ * ranges, llmc/cuda_common.h:115-124, and reads times from an ncu run, profile_gpt2cu.py). When enabled,
+ * every kernel launch of this library is bracketed by HIP events on its stream; the report aggregates
+ * by kernel family: number of launches, total milliseconds, algorithmic flops and algorithmic bytes. */
+void llmk_profile_enable(int on);
+void llmk_profile_reset(void);
+int llmk_profile_count(void);
+void llmk_profile_get(int i, char* name64, int* calls, double* ms, double* flops, double* bytes);
+
+/* ---- encoder (llmc/encoder.cuh) ---------------------------------------------------------- */
+
+/* encoder_forward, llmc/encoder.cuh:157. out[b,t,:] = wte[inp[b,t],:] + wpe[t,:] */
+void llmk_encoder_forward(void* out, const int* inp, const void* wte, const void* wpe, int B, int T, int C,
+                          void* stream);
+
+/* encoder_backward, llmc/encoder.cuh:169. dwpe[t,:] += sum_b dout[b,t,:];
+ * dwte[tok,:] += sum_{bt: inp[bt]==tok} dout[bt,:]; fp32 accumulation in ascending bt order,
+ * stochastic rounding into bf16 (plain store in fp32), no atomics.
+ *   scratch           device, >= B*T*G*20 bytes with G = ceil(C / (64 * 16/sizeof(floatX))): bucket records, then
+ *                     the position list (same layout and bound as the reference, llmc/encoder.cuh:183-184,225-226)
+ *   workload_indices  host, >= B*T ints         (reference sizes it B*T*G)
+ *   bucket_info       host, >= B*T*G * 4 ints   (reference: one int4 per bucket)
+ *   inp / inputs_cpu  the same tokens on device / host */
+void llmk_encoder_backward(void* dwte, void* dwpe, void* scratch, int* workload_indices, int* bucket_info,
+                           const void* dout, const int* inp, const int* inputs_cpu, int B, int T, int C,
+                           unsigned int seed, void* stream);
+
+/* ---- layernorm / residual (llmc/layernorm.cuh) ------------------------------------------- */
+
+/* layernorm_forward, llmc/layernorm.cuh:433. mean/rstd (fp32, B*T) may be NULL. */
+void llmk_layernorm_forward(void* out, float* mean, float* rstd, const void* inp, const void* weight,
+                            const void* bias, int B, int T, int C, void* stream);
+
+/* residual_forward, llmc/layernorm.cuh:458 */
+void llmk_residual_forward(void* out, const void* inp1, const void* inp2, int N, void* stream);
+
+/* fused_residual_forward5, llmc/layernorm.cuh:467. residual = inp1 + inp2 (rounded to floatX),
+ * normed = LN(residual). mean/rstd may be NULL. */
+void llmk_fused_residual_forward5(void* residual, void* normed, float* mean, float* rstd, const void* inp1,
+                                  const void* inp2, const void* weight, const void* bias, int N, int C,
+                                  void* stream);
+
+/* layernorm_backward, llmc/layernorm.cuh:492. dinp += ..., dweight += ..., dbias += ...
+ * scratch: device fp32, >= llmk_layernorm_backward_scratch_floats(C) floats. */
+void llmk_layernorm_backward(void* dinp, void* dweight, void* dbias, float* scratch, const void* dout,
+                             const void* inp, const void* weight, const float* mean, const float* rstd, int B,
+                             int T, int C, void* stream);
+size_t llmk_layernorm_backward_scratch_floats(int C);
+
+/* ---- matmul (llmc/matmul.cuh) ------------------------------------------------------------ */
+
+/* matmul_forward_cublaslt, llmc/matmul.cuh:231. out[B*T,OC] = inp[B*T,C] . weight[OC,C]^T + bias[OC].
+ * bias may be NULL. If pre_gelu != NULL: pre_gelu receives the pre-activation and out = gelu(pre_gelu)
+ * (gelu_fusion >= 1: in the GEMM epilogue; < 1: separate gelu kernel). */
+void llmk_matmul_forward(void* out, const void* inp, const void* weight, const void* bias, int B, int T, int C,
+                         int OC, void* stream, void* pre_gelu, int gelu_fusion);
+
+/* matmul_backward, llmc/matmul.cuh:244.
+ *   dbias[OC]   += column sums of dout          (skipped when dbias == NULL)
+ *   dinp[B*T,C]  = dout . weight                 (then *= gelu'(pre_gelu) when pre_gelu != NULL;
+ *                                                 gelu_fusion >= 2: in the epilogue, else separate kernel)
+ *   dweight[OC,C] += dout^T . inp
+ * dbias_buffer: device fp32 scratch, >= llmk_matmul_backward_bias_scratch_floats(OC) floats
+ * (may be NULL when dbias == NULL). */
+void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
+                          const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
+                          const void* pre_gelu, int gelu_fusion);
+size_t llmk_matmul_backward_bias_scratch_floats(int OC);
+
+/* ---- attention (llmc/cudnn_att.cpp; the flash path the reference takes with ENABLE_CUDNN) -- */
+
+/* attention_forward_cudnn, llmc/cudnn_att.cpp:222. Causal softmax(Q K^T / sqrt(hs)) V.
+ * inp (B,T,3,NH,hs) read in place; out (B,T,NH,hs); stats (B,NH,T) fp32 = log-sum-exp of the
+ * scaled scores of each row, NULL for inference. */
+void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int T, int NH, int C, void* stream);
+
+/* attention_backward_cudnn, llmc/cudnn_att.cpp:256. dqkvr (B,T,3,NH,hs) is overwritten.
+ * Deterministic (no atomics), as the reference requests from cuDNN (cudnn_att.cpp:187-189).
+ * Uses B*NH*T floats of the library workspace for the rowsum(dO*O) term. */
+void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
+                             int B, int T, int NH, int C, void* stream);
+
+/* ---- gelu (llmc/gelu.cuh) ----------------------------------------------------------------- */
+
+/* gelu_forward, llmc/gelu.cuh:50 */
+void llmk_gelu_forward(void* out, const void* inp, int N, void* stream);
+/* gelu_backward_inplace, llmc/gelu.cuh:59. d_in_out *= gelu'(inp) */
+void llmk_gelu_backward_inplace(void* d_in_out, const void* inp, int N, void* stream);
+
+/* ---- fused classifier (llmc/fused_classifier.cuh) ---------------------------------------- */
+
+/* fused_classifier, llmc/fused_classifier.cuh:139. Per row of logits (B*T, P), over the first V
+ * columns: losses[row] -= log softmax(row)[target]  (accumulates, like the reference's `-=` at :81);
+ * if write_dlogits: logits[row,i] = (softmax_i - [i==target]) * dloss in place for i < V.
+ * Columns [V,P) are left untouched. */
+void llmk_fused_classifier(void* logits, float* losses, float dloss, const int* targets, int B, int T, int V,
+                           int P, int write_dlogits, void* stream);
+
+/* ---- global norm (llmc/global_norm.cuh, llmc/cuda_utils.cuh) ------------------------------ */
+
+/* get_max_num_block_sums, llmc/global_norm.cuh:52 */
+int llmk_get_max_num_block_sums(const int* num_slices_all, int numel);
+/* global_norm_squared, llmc/global_norm.cuh:68. out[block] (+)= partial sums of values^2;
+ * reset != 0 zeroes out[0..max_num_block_sums) first. */
+void llmk_global_norm_squared(float* out, const void* values, size_t count, ptrdiff_t stride, int num_slices,
+                              int max_num_block_sums, int reset, void* stream);
+/* global_sum_deterministic<float>, llmc/cuda_utils.cuh:202. *result = sum(values[0..count)), one block. */
+void llmk_global_sum_deterministic(float* result, const float* values, int count, void* stream);
+
+/* ---- AdamW (llmc/adamw.cuh) --------------------------------------------------------------- */
+
+/* adamw_update, llmc/adamw.cuh:74. params/grads are floatX, m/v/master fp32; master may be NULL.
+ * The stochastic-rounding word of element i of slice s is
+ * SquirrelNoise5(i % 512 + 198491317 * ((i / 512) * 512 + s), seed): a pure function of
+ * (i, s, seed) that equals what the reference's launch geometry yields (llmc/cuda_utils.cuh:272). */
+void llmk_adamw_update(void* params_memory, float* master_params_memory, const void* grads_memory, float* m_memory,
+                       float* v_memory, size_t num_parameters, ptrdiff_t w_stride, ptrdiff_t g_stride,
+                       ptrdiff_t s_stride, int num_slices, float learning_rate, float beta1, float beta2, int t,
+                       float eps, float weight_decay, float grad_scale, unsigned int seed, void* stream);
+/* init_from_master, llmc/adamw.cuh:90. params = stochastic_round(master), same noise as above. */
+void llmk_init_from_master(void* params_memory, const float* master_params_memory, size_t num_parameters,
+                           ptrdiff_t w_stride, ptrdiff_t s_stride, int num_slices, unsigned int seed,
+                           void* stream);
+/* copy_and_cast_kernel<float, floatX> launch, llmc/cuda_utils.cuh:134 / train_gpt2.cu:1089-1094:
+ * dst[i + s*stride_dst] = (float)src[i + s*stride_src] */
+void llmk_copy_and_cast_to_f32(float* dst, const void* src, size_t n, ptrdiff_t stride_dst, ptrdiff_t stride_src,
+                               int num_slices, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LLMK_H */

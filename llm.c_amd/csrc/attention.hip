@@ -1,0 +1,625 @@
+// Causal self-attention, forward and backward, as fused flash-style kernels for gfx950.
+// Replaces the reference's cuDNN path (llmc/cudnn_att.cpp:222 forward, :256 backward):
+// QKV is read in place as (B,T,3,NH,hs), the output is (B,T,NH,hs), and the only thing kept for
+// backward is one fp32 log-sum-exp per (b,h,t). CPU definition: train_gpt2.c:271-405.
+//
+// bf16 build (head size 64). Everything is computed "transposed" so that no softmax statistic
+// ever has to cross lanes. A 32x32 MFMA accumulator gives each lane ONE column and 16 rows;
+// by computing S^T = K.Q^T the lane's column is a query, so the running max / sum / rescale
+// of the online softmax are per-lane scalars (one cross-half exchange per tile for the max).
+// The probabilities never leave registers: an accumulator, converted to bf16, already has the
+// MFMA B-operand layout (lane = non-contracted index, 8 contracted values), provided the other
+// operand is fetched in the same key order — which the transposing LDS read
+// (ds_read_b64_tr_b16) does for free. The same identity drives backward:
+//   dK/dV kernel: S = Q.K^T (lane = key), P and dS feed dV^T = dO^T.P and dK^T = Q^T.dS
+//   dQ kernel:    S^T = K.Q^T (lane = query), dS^T feeds dQ^T = K^T.dS^T
+// Two kernels instead of one with atomics: every output element has exactly one owner, so the
+// result is deterministic, as the reference requests from cuDNN (cudnn_att.cpp:187-189).
+//
+// fp32 build: straightforward one-wave-per-row kernels (lanes = head dimensions), used only for
+// parity runs against the CPU reference at small sizes.
+#include "common.hpp"
+#include "../../include/llmk.h"
+
+namespace {
+
+#if !defined(LLMK_FP32)
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+constexpr int HS = 64;
+constexpr int KP = 144;               // LDS pitch (bytes) of a [row][64 x bf16] tile: 128 + 16, conflict-free for
+                                      // both ds_read_b128 down a column of rows and the transposing 8-byte reads
+constexpr int TILE_BYTES = 64 * KP;   // 64 rows
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// rows [row0,row0+32) x k in [16s, 16s+16): MFMA operand read along K-contiguous rows
+__device__ __forceinline__ bf16x8 frag_rows(const char* tile, int row0, int s, int lane) {
+    return *reinterpret_cast<const bf16x8*>(tile + (row0 + (lane & 31)) * KP + (2 * s + (lane >> 5)) * 16);
+}
+// Transposed operand: lane (idx = lane&31, half = lane>>5) receives, for e = 0..7,
+//   tile[kbase + 8*(e/4) + 4*half + e%4][col0 + idx]
+// i.e. the contracted index runs over tile ROWS, in exactly the order in which a 32x32
+// accumulator's registers r = 8*s2 .. 8*s2+7 enumerate its rows.
+__device__ __forceinline__ bf16x8 frag_cols_accorder(const char* tile, int kbase, int col0, int lane) {
+    const int s16 = lane & 15, grp = lane >> 4;
+    const int row = kbase + 4 * (grp >> 1) + (s16 >> 2);
+    const int col = col0 + (grp & 1) * 16 + 4 * (s16 & 3);
+    const char* p = tile + row * KP + col * 2;
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p + 8 * KP));
+    union { struct { s16x4 a, b; } s; bf16x8 v; } u;
+    u.s.a = lo; u.s.b = hi;
+    return u.v;
+}
+// accumulator registers r = 8*s2 .. 8*s2+7 as a bf16 operand
+__device__ __forceinline__ bf16x8 pack_acc(const f32x16& a, int s2) {
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; e++) o[e] = (__bf16)a[8 * s2 + e];
+    return o;
+}
+// row index (within a 32-row block) of accumulator register r for this lane
+__device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
+
+// cooperative 64x64 bf16 tile copy global -> registers (2 x 16 B per thread, 256 threads)
+struct TileRegs { u32x4 v[2]; };
+__device__ __forceinline__ void tile_load(TileRegs& t, const floatX* base, size_t row_stride, int row0, int nrows, int tid) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int q = tid + i * 256, row = q >> 3, c = q & 7;
+        u32x4 z = {0, 0, 0, 0};
+        t.v[i] = (row0 + row < nrows) ? *reinterpret_cast<const u32x4*>(base + (size_t)(row0 + row) * row_stride + c * 8) : z;
+    }
+}
+__device__ __forceinline__ void tile_store(char* tile, const TileRegs& t, int tid) {
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        const int q = tid + i * 256, row = q >> 3, c = q & 7;
+        *reinterpret_cast<u32x4*>(tile + row * KP + c * 16) = t.v[i];
+    }
+}
+// 4 consecutive head-dim values of one row -> 8-byte store
+__device__ __forceinline__ void store4(floatX* p, float a, float b, float c, float d) {
+    bf16x4 o;
+    o[0] = (__bf16)a; o[1] = (__bf16)b; o[2] = (__bf16)c; o[3] = (__bf16)d;
+    *reinterpret_cast<bf16x4*>(p) = o;
+}
+
+// ---- forward ----------------------------------------------------------------------------------
+// grid (ceil(T/128), B*NH), 256 threads: wave w owns queries [128*qt + 32w, +32)
+__global__ void __launch_bounds__(256)
+fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
+    __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char sV[2][TILE_BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    const int qt = gridDim.x - 1 - blockIdx.x;          // longest rows first
+    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+    const float c = 0.125f * LOG2E;                       // 1/sqrt(64) folded into the exp2 argument
+
+    bf16x8 qf[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_q < T) qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+        else
+#pragma unroll
+            for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
+    }
+    f32x16 o[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[d][r] = 0.f;
+    float m = -INFINITY, l = 0.f;
+
+    const int last_q = min(qt * 128 + 127, T - 1);
+    const int n_kt = last_q / 64 + 1;
+    TileRegs rk, rv;
+    tile_load(rk, base + C, C3, 0, T, tid);
+    tile_load(rv, base + 2 * C, C3, 0, T, tid);
+    tile_store(sK[0], rk, tid);
+    tile_store(sV[0], rv, tid);
+    __syncthreads();
+
+    for (int j = 0; j < n_kt; j++) {
+        const char* tk = sK[j & 1];
+        const char* tv = sV[j & 1];
+        const bool more = j + 1 < n_kt;
+        if (more) {
+            tile_load(rk, base + C, C3, 64 * (j + 1), T, tid);
+            tile_load(rv, base + 2 * C, C3, 64 * (j + 1), T, tid);
+        }
+        if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
+            f32x16 sacc[2];
+            const bool kb1 = 64 * j + 32 <= qw0 + 31;     // second 32-key block not entirely masked
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[kb][r] = 0.f;
+                if (kb == 0 || kb1) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++)
+                        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32 * kb, s, lane), qf[s], sacc[kb], 0, 0, 0);
+                }
+            }
+            const bool diag = 64 * j + 63 > qw0;          // some (key, query) pairs of this tile are masked
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    if (diag) {
+                        const int key = 64 * j + 32 * kb + acc_row(r, lane);
+                        if (key > my_q) sacc[kb][r] = -INFINITY;
+                    }
+                    mx = fmaxf(mx, sacc[kb][r]);
+                }
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m, mx * c);
+            const float alpha = fast_exp2(m - m_new);
+            m = m_new;
+            float rs = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    float p = fast_exp2(fmaf(sacc[kb][r], c, -m_new));
+                    sacc[kb][r] = p;
+                    rs += p;
+                }
+            l = l * alpha + rs;
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+#pragma unroll
+            for (int s2 = 0; s2 < 4; s2++) {
+                if (s2 < 2 || kb1) {
+                    bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+                        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tv, 16 * s2, 32 * d, lane), pf, o[d], 0, 0, 0);
+                }
+            }
+        }
+        if (more) {
+            tile_store(sK[(j + 1) & 1], rk, tid);
+            tile_store(sV[(j + 1) & 1], rv, tid);
+        }
+        __syncthreads();
+    }
+
+    l += __shfl_xor(l, 32, WAVE);
+    if (my_q < T) {
+        const float inv = 1.0f / l;
+        floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                store4(dst + 32 * d + 8 * g + 4 * half, o[d][4 * g] * inv, o[d][4 * g + 1] * inv, o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+        if (stats && half == 0) stats[((size_t)b * NH + h) * T + my_q] = (m + __log2f(l)) * 0.6931471805599453f;
+    }
+}
+
+// ---- backward: D[b,h,t] = sum_d dO * O ------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+fa_dot_do_o_kernel(float* __restrict__ D, const floatX* __restrict__ dout, const floatX* __restrict__ o, int B, int T, int NH) {
+    // 8 lanes per (b,t,h) row of 64 values
+    const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t row = gid >> 3;
+    const int part = (int)(gid & 7);
+    const size_t nrows = (size_t)B * T * NH;
+    float s = 0.f;
+    if (row < nrows) {
+        vecX a = ld_vec(dout + row * HS + part * 8), bb = ld_vec(o + row * HS + part * 8);
+#pragma unroll
+        for (int k = 0; k < 8; k++) s += to_f32(a[k]) * to_f32(bb[k]);
+    }
+    s += __shfl_xor(s, 1, WAVE);
+    s += __shfl_xor(s, 2, WAVE);
+    s += __shfl_xor(s, 4, WAVE);
+    if (row < nrows && part == 0) {
+        const size_t bt = row / NH;
+        const int h = (int)(row % NH);
+        const size_t b = bt / T, t = bt % T;
+        D[(b * NH + h) * T + t] = s;
+    }
+}
+
+// ---- backward: dK, dV --------------------------------------------------------------------------------
+// grid (ceil(T/128), B*NH): wave w owns keys [128*kt + 32w, +32) and walks all later query tiles
+__global__ void __launch_bounds__(256)
+fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                        const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+    __shared__ __attribute__((aligned(16))) char sQ[2][TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char sdO[2][TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) float sL[2][64];
+    __shared__ __attribute__((aligned(16))) float sD[2][64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    const int kt = blockIdx.x;
+    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const floatX* dobase = dout + (size_t)b * T * C + h * HS;
+    const float* lbase = stats + ((size_t)b * NH + h) * T;
+    const float* dbase = Dsum + ((size_t)b * NH + h) * T;
+    const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
+    const float c = 0.125f * LOG2E;
+
+    bf16x8 kf[4], vf[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_k < T) {
+            kf[s] = *reinterpret_cast<const bf16x8*>(base + C + (size_t)my_k * C3 + 16 * s + 8 * half);
+            vf[s] = *reinterpret_cast<const bf16x8*>(base + 2 * C + (size_t)my_k * C3 + 16 * s + 8 * half);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) { kf[s][e] = (__bf16)0.f; vf[s][e] = (__bf16)0.f; }
+        }
+    }
+    f32x16 dv[2], dk[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) { dv[d][r] = 0.f; dk[d][r] = 0.f; }
+
+    const int q_first = (kt * 128) / 64, q_end = CEIL_DIV(T, 64);
+    TileRegs rq, rdo;
+    float rstat = 0.f;
+    auto load_stats = [&](int qi) {
+        const int q = 64 * qi + (tid & 63);
+        if (tid < 64) rstat = q < T ? lbase[q] * LOG2E : 0.f;
+        else if (tid < 128) rstat = q < T ? dbase[q] : 0.f;
+    };
+    auto store_stats = [&](int buf) {
+        if (tid < 64) sL[buf][tid] = rstat;
+        else if (tid < 128) sD[buf][tid - 64] = rstat;
+    };
+    if (q_first < q_end) {
+        tile_load(rq, base, C3, 64 * q_first, T, tid);
+        tile_load(rdo, dobase, (size_t)C, 64 * q_first, T, tid);
+        load_stats(q_first);
+        tile_store(sQ[0], rq, tid);
+        tile_store(sdO[0], rdo, tid);
+        store_stats(0);
+    }
+    __syncthreads();
+
+    for (int qi = q_first; qi < q_end; qi++) {
+        const int buf = (qi - q_first) & 1;
+        const char* tq = sQ[buf];
+        const char* tdo = sdO[buf];
+        const bool more = qi + 1 < q_end;
+        if (more) {
+            tile_load(rq, base, C3, 64 * (qi + 1), T, tid);
+            tile_load(rdo, dobase, (size_t)C, 64 * (qi + 1), T, tid);
+            load_stats(qi + 1);
+        }
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            const int q0 = 64 * qi + 32 * qb;
+            if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
+            f32x16 sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s, lane), vf[s], pacc, 0, 0, 0);
+            }
+            const bool diag = q0 < kw0 + 31;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int rr = 32 * qb + g * 8 + half * 4;
+                const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[buf][rr]);
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int r = 4 * g + e;
+                    float p = fast_exp2(fmaf(sacc[r], c, -l4[e]));
+                    const int q = 64 * qi + rr + e;
+                    if ((diag && q < my_k) || q >= T) p = 0.f;
+                    sacc[r] = p;
+                    pacc[r] = p * (pacc[r] - d4[e]);
+                }
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
+#pragma unroll
+                for (int d = 0; d < 2; d++) {
+                    dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tdo, 32 * qb + 16 * s2, 32 * d, lane), pf, dv[d], 0, 0, 0);
+                    dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tq, 32 * qb + 16 * s2, 32 * d, lane), dsf, dk[d], 0, 0, 0);
+                }
+            }
+        }
+        if (more) {
+            tile_store(sQ[buf ^ 1], rq, tid);
+            tile_store(sdO[buf ^ 1], rdo, tid);
+            store_stats(buf ^ 1);
+        }
+        __syncthreads();
+    }
+
+    if (my_k < T) {
+        floatX* dkp = dqkv + ((size_t)b * T + my_k) * C3 + C + h * HS;
+        floatX* dvp = dqkv + ((size_t)b * T + my_k) * C3 + 2 * C + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int col = 32 * d + 8 * g + 4 * half;
+                store4(dkp + col, dk[d][4 * g] * 0.125f, dk[d][4 * g + 1] * 0.125f, dk[d][4 * g + 2] * 0.125f, dk[d][4 * g + 3] * 0.125f);
+                store4(dvp + col, dv[d][4 * g], dv[d][4 * g + 1], dv[d][4 * g + 2], dv[d][4 * g + 3]);
+            }
+    }
+}
+
+// ---- backward: dQ ---------------------------------------------------------------------------------------
+// grid (ceil(T/128), B*NH): wave w owns queries [128*qt + 32w, +32) and walks the key tiles up to the diagonal
+__global__ void __launch_bounds__(256)
+fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                      const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+    __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
+    __shared__ __attribute__((aligned(16))) char sV[2][TILE_BYTES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    const int qt = gridDim.x - 1 - blockIdx.x;
+    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+    const float c = 0.125f * LOG2E;
+
+    bf16x8 qf[4], dof[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_q < T) {
+            qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+            dof[s] = *reinterpret_cast<const bf16x8*>(dout + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) { qf[s][e] = (__bf16)0.f; dof[s][e] = (__bf16)0.f; }
+        }
+    }
+    const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
+    const float dsum = my_q < T ? Dsum[((size_t)b * NH + h) * T + my_q] : 0.f;
+    f32x16 dq[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dq[d][r] = 0.f;
+
+    const int last_q = min(qt * 128 + 127, T - 1);
+    const int n_kt = last_q / 64 + 1;
+    TileRegs rk, rv;
+    tile_load(rk, base + C, C3, 0, T, tid);
+    tile_load(rv, base + 2 * C, C3, 0, T, tid);
+    tile_store(sK[0], rk, tid);
+    tile_store(sV[0], rv, tid);
+    __syncthreads();
+
+    for (int j = 0; j < n_kt; j++) {
+        const char* tk = sK[j & 1];
+        const char* tv = sV[j & 1];
+        const bool more = j + 1 < n_kt;
+        if (more) {
+            tile_load(rk, base + C, C3, 64 * (j + 1), T, tid);
+            tile_load(rv, base + 2 * C, C3, 64 * (j + 1), T, tid);
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const int k0 = 64 * j + 32 * kb;
+            if (k0 > qw0 + 31) continue;
+            f32x16 sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32 * kb, s, lane), qf[s], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tv, 32 * kb, s, lane), dof[s], pacc, 0, 0, 0);
+            }
+            const bool diag = k0 + 31 > qw0;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                float p = fast_exp2(fmaf(sacc[r], c, -lse2));
+                if (diag && (k0 + acc_row(r, lane) > my_q)) p = 0.f;
+                pacc[r] = p * (pacc[r] - dsum);
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const bf16x8 dsf = pack_acc(pacc, s2);
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+                    dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tk, 32 * kb + 16 * s2, 32 * d, lane), dsf, dq[d], 0, 0, 0);
+            }
+        }
+        if (more) {
+            tile_store(sK[(j + 1) & 1], rk, tid);
+            tile_store(sV[(j + 1) & 1], rv, tid);
+        }
+        __syncthreads();
+    }
+    if (my_q < T) {
+        floatX* dqp = dqkv + ((size_t)b * T + my_q) * C3 + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                store4(dqp + 32 * d + 8 * g + 4 * half, dq[d][4 * g] * 0.125f, dq[d][4 * g + 1] * 0.125f, dq[d][4 * g + 2] * 0.125f,
+                       dq[d][4 * g + 3] * 0.125f);
+    }
+}
+
+#else
+// =============================================================================================
+// fp32 build: one wavefront per row, lanes = head dimensions (hs <= 64)
+// =============================================================================================
+__global__ void __launch_bounds__(256)
+att_forward_f32_kernel(float* __restrict__ out, float* __restrict__ stats, const float* __restrict__ qkv, int B, int T,
+                       int NH, int hs) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);       // (b, h, t)
+    if (row >= (size_t)B * NH * T) return;
+    const int t = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
+    const int C = NH * hs;
+    const size_t C3 = 3 * (size_t)C;
+    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const float scale = 1.0f / sqrtf((float)hs);
+    const bool act = lane < hs;
+    const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
+    float m = -INFINITY, l = 0.f, acc = 0.f;
+    for (int t2 = 0; t2 <= t; t2++) {
+        const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
+        const float s = wave_sum(q * k) * scale;
+        const float m_new = fmaxf(m, s);
+        const float alpha = expf(m - m_new), p = expf(s - m_new);
+        const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
+        acc = acc * alpha + p * v;
+        l = l * alpha + p;
+        m = m_new;
+    }
+    if (act) out[((size_t)b * T + t) * C + h * hs + lane] = acc / l;
+    if (stats && lane == 0) stats[((size_t)b * NH + h) * T + t] = m + logf(l);
+}
+
+// dQ: one wave per query row
+__global__ void __launch_bounds__(256)
+att_backward_dq_f32_kernel(float* __restrict__ dqkv, const float* __restrict__ dout, const float* __restrict__ qkv,
+                           const float* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (size_t)B * NH * T) return;
+    const int t = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
+    const int C = NH * hs;
+    const size_t C3 = 3 * (size_t)C;
+    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const float scale = 1.0f / sqrtf((float)hs);
+    const bool act = lane < hs;
+    const size_t orow = ((size_t)b * T + t) * C + h * hs;
+    const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
+    const float go = act ? dout[orow + lane] : 0.f;
+    const float dsum = wave_sum(act ? go * o[orow + lane] : 0.f);
+    const float lse = stats[((size_t)b * NH + h) * T + t];
+    float dq = 0.f;
+    for (int t2 = 0; t2 <= t; t2++) {
+        const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
+        const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
+        const float s = wave_sum(q * k) * scale;
+        const float dp = wave_sum(go * v);
+        const float p = expf(s - lse);
+        dq += p * (dp - dsum) * scale * k;
+    }
+    if (act) dqkv[((size_t)b * T + t) * C3 + h * hs + lane] = dq;
+}
+
+// dK, dV: one wave per key row
+__global__ void __launch_bounds__(256)
+att_backward_dkdv_f32_kernel(float* __restrict__ dqkv, const float* __restrict__ dout, const float* __restrict__ qkv,
+                             const float* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
+    const int lane = threadIdx.x & 63;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= (size_t)B * NH * T) return;
+    const int t2 = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
+    const int C = NH * hs;
+    const size_t C3 = 3 * (size_t)C;
+    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const float scale = 1.0f / sqrtf((float)hs);
+    const bool act = lane < hs;
+    const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
+    const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
+    float dk = 0.f, dv = 0.f;
+    for (int t = t2; t < T; t++) {
+        const size_t orow = ((size_t)b * T + t) * C + h * hs;
+        const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
+        const float go = act ? dout[orow + lane] : 0.f;
+        const float dsum = wave_sum(act ? go * o[orow + lane] : 0.f);
+        const float s = wave_sum(q * k) * scale;
+        const float dp = wave_sum(go * v);
+        const float p = expf(s - stats[((size_t)b * NH + h) * T + t]);
+        dv += p * go;
+        dk += p * (dp - dsum) * scale * q;
+    }
+    if (act) {
+        dqkv[((size_t)b * T + t2) * C3 + C + h * hs + lane] = dk;
+        dqkv[((size_t)b * T + t2) * C3 + 2 * C + h * hs + lane] = dv;
+    }
+}
+#endif
+
+}  // namespace
+
+extern "C" {
+
+void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int T, int NH, int C, void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(NH > 0 && C % NH == 0, "attention_forward: C=%d not divisible by NH=%d", C, NH);
+    const int hs = C / NH;
+    if ((size_t)B * T == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
+    llmk::ProfScope prof("attention_forward", fwd_flops, 4.0 * B * T * C * sizeof(floatX), st);
+#if !defined(LLMK_FP32)
+    LLMK_REQUIRE(hs == HS, "attention_forward: head size %d unsupported (bf16 build handles 64)", hs);
+    LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
+    fa_forward_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+#else
+    LLMK_REQUIRE(hs <= 64, "attention_forward: head size %d unsupported (fp32 build handles <= 64)", hs);
+    const size_t rows = (size_t)B * NH * T;
+    att_forward_f32_kernel<<<(unsigned)CEIL_DIV(rows, (size_t)4), 256, 0, st>>>((float*)out, stats, (const float*)inp, B, T, NH, hs);
+#endif
+    LAUNCH_CHECK();
+}
+
+void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
+                             int B, int T, int NH, int C, void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(NH > 0 && C % NH == 0, "attention_backward: C=%d not divisible by NH=%d", C, NH);
+    LLMK_REQUIRE(stats != nullptr, "attention_backward: stats from the forward pass are required");
+    const int hs = C / NH;
+    if ((size_t)B * T == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+#if !defined(LLMK_FP32)
+    LLMK_REQUIRE(hs == HS, "attention_backward: head size %d unsupported (bf16 build handles 64)", hs);
+    float* Dsum = (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
+    const size_t nrows = (size_t)B * T * NH;
+    const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
+    {
+        llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
+        fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
+        LAUNCH_CHECK();
+    }
+    dim3 grid(CEIL_DIV(T, 128), B * NH);
+    {   // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x here, 1.0x on dQ
+        llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+        fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+        LAUNCH_CHECK();
+    }
+    llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
+    fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+    LAUNCH_CHECK();
+#else
+    LLMK_REQUIRE(hs <= 64, "attention_backward: head size %d unsupported (fp32 build handles <= 64)", hs);
+    const size_t rows = (size_t)B * NH * T;
+    const unsigned blocks = (unsigned)CEIL_DIV(rows, (size_t)4);
+    att_backward_dq_f32_kernel<<<blocks, 256, 0, st>>>((float*)dqkvr, (const float*)dout, (const float*)qkvr, (const float*)o, stats, B, T, NH, hs);
+    LAUNCH_CHECK();
+    att_backward_dkdv_f32_kernel<<<blocks, 256, 0, st>>>((float*)dqkvr, (const float*)dout, (const float*)qkvr, (const float*)o, stats, B, T, NH, hs);
+    LAUNCH_CHECK();
+#endif
+}
+
+}  // extern "C"

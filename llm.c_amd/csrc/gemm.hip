@@ -1,0 +1,582 @@
+// Dense contractions of the GPT-2 step on gfx950 matrix cores: matmul_forward / matmul_backward
+// (reference launchers llmc/matmul.cuh:231 and :244, which hand the work to cuBLASLt; CPU
+// definition train_gpt2.c:163-269).
+//
+//   forward   out[M,OC]  = inp[M,C] . W[OC,C]^T (+bias) (+GELU)      "NT": both operands K-contiguous
+//   dinp      dinp[M,C]  = dout[M,OC] . W[OC,C]      (* gelu')        "NN": B stored K-major
+//   dweight   dW[OC,C]  += dout[M,OC]^T . inp[M,C]                    "TN": both stored K-major, K = M = B*T
+//
+// bf16 build: one kernel template. A workgroup owns a BM x BN tile of C and walks K in steps
+// of 64: global -> registers -> LDS (double-buffered, one barrier per step), LDS -> MFMA
+// operands, v_mfma_f32_32x32x16_bf16 with fp32 accumulators.
+//   * K-contiguous operands sit in LDS as [row][64] with the eight 16-byte chunks of a row
+//     XOR-swizzled by (row & 7): both the 16-byte writes and the ds_read_b128 operand reads
+//     are bank-conflict free without padding.
+//   * K-major operands (the weight in dinp, both operands in dweight) sit in LDS as they are
+//     in memory, [k][row] with a padded pitch, and are turned into MFMA operand layout by the
+//     gfx950 transposing LDS read (ds_read_b64_tr_b16): 16 lanes fetch a 4(k) x 16(row) patch
+//     and each lane receives the 4 k-values of its row. No software transpose anywhere.
+//   * Workgroup ids are remapped so that consecutive tiles land on the same XCD (ids are dealt
+//     round-robin over the 8 XCDs, each with a private L2) and walk the tile grid in groups of
+//     8 row-tiles, so an XCD's 32 resident tiles share operand panels through its L2.
+//   * dweight has few output tiles (27 for 2304x768) but K = 65536: the contraction is split
+//     over workgroups, partials go to the library workspace in fp32 and are added in split
+//     order by a second kernel (deterministic; no atomics), which also does the += into dW.
+// fp32 build: same structure with v_mfma_f32_32x32x2_f32 (true fp32 multiply-add), the mode
+// used for 1e-5 parity against the CPU reference.
+#include "common.hpp"
+#include "gelu.hpp"
+#include "../../include/llmk.h"
+
+namespace {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
+
+enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5 };
+
+struct GemmArgs {
+    const floatX* A;
+    const floatX* B;
+    floatX* C;
+    int M, N, K;          // C[M][N] = sum_k A(m,k) * B(n,k)
+    int lda, ldb, ldc;    // leading dimensions of the stored matrices, in elements
+    const floatX* bias;   // [N] or nullptr                         (EPI_BIAS*)
+    floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU)
+    float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL)
+    int k_per_split;      // multiple of the K step
+};
+
+constexpr int GROUP_M = 8;
+
+__device__ __forceinline__ void tile_coords(int tiles_m, int tiles_n, int& tm, int& tn) {
+    int pid = blockIdx.x;
+    const int nblk = gridDim.x;
+    if ((nblk & 7) == 0) pid = (pid & 7) * (nblk >> 3) + (pid >> 3);   // same-XCD ids become consecutive
+    const int per_group = GROUP_M * tiles_n;
+    const int group = pid / per_group;
+    const int first_m = group * GROUP_M;
+    const int gsz = min(tiles_m - first_m, GROUP_M);
+    const int in_group = pid - group * per_group;
+    tm = first_m + in_group % gsz;
+    tn = in_group / gsz;
+}
+
+template <int EPI>
+__device__ __forceinline__ void epilogue_store(const GemmArgs& g, int m, int n, float v, float bias_n) {
+    const size_t idx = (size_t)m * g.ldc + n;
+    if (EPI == EPI_BIAS) {
+        g.C[idx] = from_f32<floatX>(v + bias_n);
+    } else if (EPI == EPI_BIAS_GELU) {
+        floatX pre = from_f32<floatX>(v + bias_n);
+        g.aux[idx] = pre;
+        g.C[idx] = from_f32<floatX>(gelu_f(to_f32(pre)));   // GELU of the rounded pre-activation, as a separate kernel would see it
+    } else if (EPI == EPI_STORE) {
+        g.C[idx] = from_f32<floatX>(v);
+    } else if (EPI == EPI_DGELU) {
+        g.C[idx] = from_f32<floatX>(gelu_grad_f(to_f32(g.aux[idx])) * to_f32(from_f32<floatX>(v)));
+    } else if (EPI == EPI_ACCUM) {
+        g.C[idx] = from_f32<floatX>(to_f32(g.C[idx]) + v);
+    } else {
+        g.partial[((size_t)blockIdx.y * g.M + m) * g.N + n] = v;
+    }
+}
+
+#if !defined(LLMK_FP32)
+// =============================================================================================
+// bf16 MFMA kernel
+// =============================================================================================
+constexpr int BK = 64;
+
+template <int R, bool TRANS> struct TileLayout;
+template <int R> struct TileLayout<R, false> {           // [R][64] bf16, chunk-swizzled
+    static constexpr int BYTES = R * 128;
+};
+template <int R> struct TileLayout<R, true> {            // [64][R] bf16, padded pitch
+    static constexpr int PITCH = R * 2 + 64;
+    static constexpr int BYTES = 64 * PITCH;
+};
+
+// Per-thread description of the 16-byte chunks it moves for one operand tile.
+template <int R, bool TRANS, int NT>
+struct Loader {
+    static constexpr int NCH = R * 8 / NT;               // chunks per thread
+    const floatX* gptr[NCH];                             // address at k0 = 0 (or nullptr-equivalent when masked)
+    int lds_off[NCH];
+    bool ok[NCH];
+    int kidx[NCH];                                       // k offset of the chunk inside the tile (for the K tail)
+    size_t kstride;                                      // elements to advance per K step
+
+    __device__ __forceinline__ void init(const floatX* base, int ld, int r0, int rmax, int tid) {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const int q = tid + i * NT;
+            if (!TRANS) {
+                const int row = q >> 3, c = q & 7;
+                ok[i] = (r0 + row) < rmax;
+                gptr[i] = base + (size_t)(r0 + row) * ld + c * 8;
+                lds_off[i] = row * 128 + ((c ^ (row & 7)) << 4);
+                kidx[i] = c * 8;
+            } else {
+                constexpr int CPR = R / 8;               // chunks per k-row
+                const int krow = q / CPR, cc = q % CPR;
+                ok[i] = (r0 + cc * 8) < rmax;
+                gptr[i] = base + (size_t)krow * ld + r0 + cc * 8;
+                lds_off[i] = krow * TileLayout<R, true>::PITCH + cc * 16;
+                kidx[i] = krow;
+            }
+        }
+        kstride = TRANS ? (size_t)BK * ld : (size_t)BK;
+    }
+    __device__ __forceinline__ void load(u32x4 (&reg)[NCH], int kt, int k0, int kend) const {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) {
+            const bool p = ok[i] && (k0 + kidx[i] < kend);
+            u32x4 z = {0, 0, 0, 0};
+            reg[i] = p ? *reinterpret_cast<const u32x4*>(gptr[i] + (size_t)kt * kstride) : z;
+        }
+    }
+    __device__ __forceinline__ void store(char* lds, const u32x4 (&reg)[NCH]) const {
+#pragma unroll
+        for (int i = 0; i < NCH; i++) *reinterpret_cast<u32x4*>(lds + lds_off[i]) = reg[i];
+    }
+};
+
+// MFMA operand (32 rows x 16 k) for k-step s of the tile, rows [row0, row0+32)
+template <int R, bool TRANS>
+__device__ __forceinline__ bf16x8 read_frag(const char* lds, int row0, int s, int lane) {
+    if (!TRANS) {
+        const int row = row0 + (lane & 31);
+        const int c = 2 * s + (lane >> 5);
+        return *reinterpret_cast<const bf16x8*>(lds + row * 128 + ((c ^ (row & 7)) << 4));
+    } else {
+        constexpr int PITCH = TileLayout<R, true>::PITCH;
+        const int s16 = lane & 15, grp = lane >> 4;
+        const int krow = 16 * s + 8 * (grp >> 1) + (s16 >> 2);
+        const int col = row0 + (grp & 1) * 16 + 4 * (s16 & 3);
+        const char* p = lds + krow * PITCH + col * 2;
+        typedef s16x4 __attribute__((address_space(3))) * lds_s16x4_ptr;
+        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p));
+        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_ptr)(p + 4 * PITCH));
+        union { struct { s16x4 a, b; } s; bf16x8 v; } u;
+        u.s.a = lo; u.s.b = hi;
+        return u.v;
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
+__global__ void __launch_bounds__(WGM * WGN * 64)
+gemm_bf16_kernel(GemmArgs g) {
+    constexpr int NT = WGM * WGN * 64;
+    constexpr int WTM = BM / WGM, WTN = BN / WGN;
+    constexpr int TM = WTM / 32, TN = WTN / 32;
+    constexpr int A_BYTES = TileLayout<BM, A_T>::BYTES, B_BYTES = TileLayout<BN, B_T>::BYTES;
+    constexpr int STAGE = A_BYTES + B_BYTES;
+    extern __shared__ __attribute__((aligned(16))) char lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave / WGN, wn = wave % WGN;
+    int tile_m, tile_n;
+    tile_coords(CEIL_DIV(g.M, BM), CEIL_DIV(g.N, BN), tile_m, tile_n);
+    const int m0 = tile_m * BM, n0 = tile_n * BN;
+    const int kbeg = blockIdx.y * g.k_per_split;
+    const int kend = min(g.K, kbeg + g.k_per_split);
+    const int KT = CEIL_DIV(kend - kbeg, BK);
+
+    Loader<BM, A_T, NT> la;
+    Loader<BN, B_T, NT> lb;
+    la.init(g.A + (A_T ? (size_t)kbeg * g.lda : (size_t)kbeg), g.lda, m0, g.M, tid);
+    lb.init(g.B + (B_T ? (size_t)kbeg * g.ldb : (size_t)kbeg), g.ldb, n0, g.N, tid);
+
+    f32x16 acc[TM][TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++)
+#pragma unroll
+        for (int j = 0; j < TN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    u32x4 ra[Loader<BM, A_T, NT>::NCH], rb[Loader<BN, B_T, NT>::NCH];
+    if (KT > 0) {
+        la.load(ra, 0, kbeg, kend);
+        lb.load(rb, 0, kbeg, kend);
+        la.store(lds, ra);
+        lb.store(lds + A_BYTES, rb);
+    }
+    __syncthreads();
+
+    for (int kt = 0; kt < KT; kt++) {
+        const char* cur = lds + (kt & 1) * STAGE;
+        char* nxt = lds + ((kt + 1) & 1) * STAGE;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            la.load(ra, kt + 1, kbeg + (kt + 1) * BK, kend);
+            lb.load(rb, kt + 1, kbeg + (kt + 1) * BK, kend);
+        }
+#pragma unroll
+        for (int s = 0; s < BK / 16; s++) {
+            bf16x8 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; i++) fa[i] = read_frag<BM, A_T>(cur, wm * WTM + i * 32, s, lane);
+#pragma unroll
+            for (int j = 0; j < TN; j++) fb[j] = read_frag<BN, B_T>(cur + A_BYTES, wn * WTN + j * 32, s, lane);
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            la.store(nxt, ra);
+            lb.store(nxt + A_BYTES, rb);
+        }
+        __syncthreads();
+    }
+
+    // epilogue: lane holds column (lane & 31) and rows (r/4)*8 + (lane>>5)*4 + r%4 of each 32x32 tile
+#pragma unroll
+    for (int j = 0; j < TN; j++) {
+        const int n = n0 + wn * WTN + j * 32 + (lane & 31);
+        if (n >= g.N) continue;
+        float bias_n = 0.f;
+        if ((EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) && g.bias) bias_n = to_f32(g.bias[n]);
+#pragma unroll
+        for (int i = 0; i < TM; i++) {
+            const int mb = m0 + wm * WTM + i * 32 + (lane >> 5) * 4;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = mb + (r >> 2) * 8 + (r & 3);
+                if (m < g.M) epilogue_store<EPI>(g, m, n, acc[i][j][r], bias_n);
+            }
+        }
+    }
+}
+
+template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
+void launch_bf16(const GemmArgs& g, int splits, hipStream_t st) {
+    constexpr int SMEM = 2 * (TileLayout<BM, A_T>::BYTES + TileLayout<BN, B_T>::BYTES);
+    auto kern = gemm_bf16_kernel<BM, BN, WGM, WGN, A_T, B_T, EPI>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM));
+        attr_set = true;
+    }
+    dim3 grid(CEIL_DIV(g.M, BM) * CEIL_DIV(g.N, BN), splits);
+    kern<<<grid, WGM * WGN * 64, SMEM, st>>>(g);
+    LAUNCH_CHECK();
+}
+
+template <bool A_T, bool B_T, int EPI>
+void launch_gemm(const GemmArgs& g, int splits, bool big, hipStream_t st) {
+    if (big) launch_bf16<256, 256, 2, 4, A_T, B_T, EPI>(g, splits, st);
+    else launch_bf16<128, 128, 2, 2, A_T, B_T, EPI>(g, splits, st);
+}
+constexpr int K_ALIGN = 8;       // K-contiguous rows are read in 16-byte chunks
+constexpr int BIG_TILE = 256, SMALL_TILE = 128, K_STEP = 64;
+
+#else
+// =============================================================================================
+// fp32 MFMA kernel (parity mode): 128x128 tile, K step 16, 4 waves of 64x64
+// =============================================================================================
+constexpr int FBM = 128, FBN = 128, FBK = 16;
+constexpr int F_PITCH_K = FBK + 4;       // [row][k] tiles, 16-byte aligned rows
+constexpr int F_PITCH_T = 128 + 4;       // [k][row] tiles
+
+template <bool A_T, bool B_T, int EPI>
+__global__ void __launch_bounds__(256)
+gemm_f32_kernel(GemmArgs g) {
+    __shared__ __attribute__((aligned(16))) float sA[2][A_T ? FBK * F_PITCH_T : FBM * F_PITCH_K];
+    __shared__ __attribute__((aligned(16))) float sB[2][B_T ? FBK * F_PITCH_T : FBN * F_PITCH_K];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    int tile_m, tile_n;
+    tile_coords(CEIL_DIV(g.M, FBM), CEIL_DIV(g.N, FBN), tile_m, tile_n);
+    const int m0 = tile_m * FBM, n0 = tile_n * FBN;
+    const int kbeg = blockIdx.y * g.k_per_split;
+    const int kend = min(g.K, kbeg + g.k_per_split);
+    const int KT = CEIL_DIV(kend - kbeg, FBK);
+
+    // each thread moves 2 float4 per operand tile (128*16/4 = 512 float4)
+    auto load_tile = [&](const float* base, int ld, bool trans, int r0, int rmax, int k0, vecF (&reg)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int q = tid + i * 256;
+            vecF z; z[0] = z[1] = z[2] = z[3] = 0.f;
+            if (!trans) {
+                const int row = q >> 2, c = (q & 3) * 4;
+                const bool p = (r0 + row < rmax) && (k0 + c < kend);
+                reg[i] = p ? ld_vec(base + (size_t)(r0 + row) * ld + k0 + c) : z;
+            } else {
+                const int krow = q >> 5, c = (q & 31) * 4;
+                const bool p = (k0 + krow < kend) && (r0 + c < rmax);
+                reg[i] = p ? ld_vec(base + (size_t)(k0 + krow) * ld + r0 + c) : z;
+            }
+        }
+    };
+    auto store_tile = [&](float* s, bool trans, const vecF (&reg)[2]) {
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int q = tid + i * 256;
+            if (!trans) st_vec(s + (q >> 2) * F_PITCH_K + (q & 3) * 4, reg[i]);
+            else st_vec(s + (q >> 5) * F_PITCH_T + (q & 31) * 4, reg[i]);
+        }
+    };
+
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+    vecF ra[2], rb[2];
+    if (KT > 0) {
+        load_tile(g.A, g.lda, A_T, m0, g.M, kbeg, ra);
+        load_tile(g.B, g.ldb, B_T, n0, g.N, kbeg, rb);
+        store_tile(sA[0], A_T, ra);
+        store_tile(sB[0], B_T, rb);
+    }
+    __syncthreads();
+    for (int kt = 0; kt < KT; kt++) {
+        const int cur = kt & 1;
+        const bool more = kt + 1 < KT;
+        if (more) {
+            load_tile(g.A, g.lda, A_T, m0, g.M, kbeg + (kt + 1) * FBK, ra);
+            load_tile(g.B, g.ldb, B_T, n0, g.N, kbeg + (kt + 1) * FBK, rb);
+        }
+#pragma unroll
+        for (int s = 0; s < FBK / 2; s++) {
+            const int k = 2 * s + (lane >> 5);
+            float fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                const int row = wm * 64 + i * 32 + (lane & 31);
+                fa[i] = A_T ? sA[cur][k * F_PITCH_T + row] : sA[cur][row * F_PITCH_K + k];
+            }
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                const int row = wn * 64 + j * 32 + (lane & 31);
+                fb[j] = B_T ? sB[cur][k * F_PITCH_T + row] : sB[cur][row * F_PITCH_K + k];
+            }
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i], fb[j], acc[i][j], 0, 0, 0);
+        }
+        if (more) {
+            store_tile(sA[cur ^ 1], A_T, ra);
+            store_tile(sB[cur ^ 1], B_T, rb);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int j = 0; j < 2; j++) {
+        const int n = n0 + wn * 64 + j * 32 + (lane & 31);
+        if (n >= g.N) continue;
+        float bias_n = 0.f;
+        if ((EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) && g.bias) bias_n = g.bias[n];
+#pragma unroll
+        for (int i = 0; i < 2; i++) {
+            const int mb = m0 + wm * 64 + i * 32 + (lane >> 5) * 4;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int m = mb + (r >> 2) * 8 + (r & 3);
+                if (m < g.M) epilogue_store<EPI>(g, m, n, acc[i][j][r], bias_n);
+            }
+        }
+    }
+}
+
+template <bool A_T, bool B_T, int EPI>
+void launch_gemm(const GemmArgs& g, int splits, bool /*big*/, hipStream_t st) {
+    dim3 grid(CEIL_DIV(g.M, FBM) * CEIL_DIV(g.N, FBN), splits);
+    gemm_f32_kernel<A_T, B_T, EPI><<<grid, 256, 0, st>>>(g);
+    LAUNCH_CHECK();
+}
+constexpr int K_ALIGN = 4;
+constexpr int BIG_TILE = 128, SMALL_TILE = 128, K_STEP = 16;
+#endif
+
+// C[m][n] (+)= sum over splits of partial[s][m][n], in split order
+template <bool ACCUM>
+__global__ void __launch_bounds__(256)
+splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, size_t mn, int splits) {
+    size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+    if (i >= mn) return;
+    vecF s = ld_vec(partial + i);
+    for (int k = 1; k < splits; k++) {
+        vecF p = ld_vec(partial + (size_t)k * mn + i);
+#pragma unroll
+        for (int e = 0; e < 4; e++) s[e] += p[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        float base = ACCUM ? to_f32(C[i + e]) : 0.f;
+        C[i + e] = from_f32<floatX>(base + s[e]);
+    }
+}
+
+// ---- bias gradient: column sums of dout[N][OC] -----------------------------------------------
+// workgroup = 32 column-vectors x 8 row lanes; grid.y splits the rows so the machine is full.
+constexpr int VN = vecX::N;
+constexpr int BG_COLV = 32, BG_ROWL = 8;
+__global__ void __launch_bounds__(256)
+bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, int N, int OC) {
+    __shared__ float red[BG_ROWL][BG_COLV * VN + 1];
+    const int cv = threadIdx.x % BG_COLV, rl = threadIdx.x / BG_COLV;
+    const int col = (blockIdx.x * BG_COLV + cv) * VN;
+    float acc[VN];
+#pragma unroll
+    for (int k = 0; k < VN; k++) acc[k] = 0.f;
+    if (col < OC) {
+        for (int r = blockIdx.y * BG_ROWL + rl; r < N; r += gridDim.y * BG_ROWL) {
+            vecX d = ld_vec(dout + (size_t)r * OC + col);
+#pragma unroll
+            for (int k = 0; k < VN; k++) acc[k] += to_f32(d[k]);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VN; k++) red[rl][cv * VN + k] = acc[k];
+    __syncthreads();
+    for (int c = threadIdx.x; c < BG_COLV * VN; c += 256) {
+        const int oc = blockIdx.x * BG_COLV * VN + c;
+        if (oc < OC) {
+            float s = 0.f;
+#pragma unroll
+            for (int r = 0; r < BG_ROWL; r++) s += red[r][c];
+            partial[(size_t)blockIdx.y * OC + oc] = s;
+        }
+    }
+}
+__global__ void __launch_bounds__(256)
+bias_grad_reduce_kernel(floatX* __restrict__ dbias, const float* __restrict__ partial, int OC, int ny) {
+    int oc = blockIdx.x * blockDim.x + threadIdx.x;
+    if (oc >= OC) return;
+    float s = 0.f;
+    for (int y = 0; y < ny; y++) s += partial[(size_t)y * OC + oc];
+    dbias[oc] = from_f32<floatX>(to_f32(dbias[oc]) + s);
+}
+int bias_grad_ny(int OC) {
+    int gx = CEIL_DIV(OC, BG_COLV * VN);
+    return max(1, llmk::device_info().num_cu * 4 / gx);
+}
+
+bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+void llmk_matmul_forward(void* out, const void* inp, const void* weight, const void* bias, int B, int T, int C,
+                         int OC, void* stream, void* pre_gelu, int gelu_fusion) {
+    if (llmk::failed()) return;
+    const int M = B * T;
+    LLMK_REQUIRE(C % K_ALIGN == 0, "matmul_forward: C=%d must be a multiple of %d", C, K_ALIGN);
+    LLMK_REQUIRE(aligned16(inp) && aligned16(weight), "matmul_forward: operands must be 16-byte aligned");
+    if (M == 0 || OC == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    GemmArgs g{};
+    g.A = (const floatX*)inp; g.B = (const floatX*)weight; g.M = M; g.N = OC; g.K = C;
+    g.lda = C; g.ldb = C; g.ldc = OC; g.bias = (const floatX*)bias; g.k_per_split = CEIL_DIV(C, K_STEP) * K_STEP;
+    const int num_cu = llmk::device_info().num_cu;
+    const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(OC, BIG_TILE) >= (size_t)num_cu;
+    llmk::ProfScope prof((pre_gelu && gelu_fusion >= 1) ? "gemm_nt_gelu" : "gemm_nt", 2.0 * M * (double)OC * C,
+                         ((double)M * C + (double)OC * C + (double)M * OC) * sizeof(floatX), st);
+    if (pre_gelu && gelu_fusion >= 1) {
+        g.C = (floatX*)out; g.aux = (floatX*)pre_gelu;
+        launch_gemm<false, false, EPI_BIAS_GELU>(g, 1, big, st);
+    } else if (pre_gelu) {
+        g.C = (floatX*)pre_gelu;
+        launch_gemm<false, false, EPI_BIAS>(g, 1, big, st);
+        if (prof.on) { llmk::prof_end(st); prof.on = false; }
+        llmk_gelu_forward(out, pre_gelu, M * OC, stream);
+    } else {
+        g.C = (floatX*)out;
+        launch_gemm<false, false, EPI_BIAS>(g, 1, big, st);
+    }
+}
+
+size_t llmk_matmul_backward_bias_scratch_floats(int OC) { return (size_t)bias_grad_ny(OC) * OC; }
+
+void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
+                          const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
+                          const void* pre_gelu, int gelu_fusion) {
+    if (llmk::failed()) return;
+    const int M = B * T;
+    LLMK_REQUIRE(C % 8 == 0 && OC % 8 == 0, "matmul_backward: C=%d and OC=%d must be multiples of 8", C, OC);
+    LLMK_REQUIRE(aligned16(dout) && aligned16(inp) && aligned16(weight), "matmul_backward: operands must be 16-byte aligned");
+    if (M == 0 || OC == 0 || C == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    const int num_cu = llmk::device_info().num_cu;
+
+    // (1) dbias += column sums of dout
+    if (dbias) {
+        LLMK_REQUIRE(dbias_buffer != nullptr, "matmul_backward: dbias_buffer is required when dbias is given");
+        const int ny = bias_grad_ny(OC);
+        llmk::ProfScope prof("bias_grad", 0, (double)M * OC * sizeof(floatX), st);
+        bias_grad_kernel<<<dim3(CEIL_DIV(OC, BG_COLV * VN), ny), 256, 0, st>>>(dbias_buffer, (const floatX*)dout, M, OC);
+        LAUNCH_CHECK();
+        bias_grad_reduce_kernel<<<CEIL_DIV(OC, 256), 256, 0, st>>>((floatX*)dbias, dbias_buffer, OC, ny);
+        LAUNCH_CHECK();
+    }
+
+    // (2) dinp[M,C] = dout[M,OC] . W[OC,C]   (A = dout K-contiguous, B(n=c,k=oc) stored [k][n])
+    {
+        GemmArgs g{};
+        g.A = (const floatX*)dout; g.B = (const floatX*)weight; g.C = (floatX*)dinp;
+        g.M = M; g.N = C; g.K = OC; g.lda = OC; g.ldb = C; g.ldc = C;
+        g.k_per_split = CEIL_DIV(OC, K_STEP) * K_STEP;
+        const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(C, BIG_TILE) >= (size_t)num_cu;
+        const bool fused = pre_gelu && gelu_fusion >= 2;
+        {
+            llmk::ProfScope prof(fused ? "gemm_nn_dgelu" : "gemm_nn", 2.0 * M * (double)OC * C,
+                                 ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
+            if (fused) {
+                g.aux = (floatX*)pre_gelu;
+                launch_gemm<false, true, EPI_DGELU>(g, 1, big, st);
+            } else {
+                launch_gemm<false, true, EPI_STORE>(g, 1, big, st);
+            }
+        }
+        if (pre_gelu && !fused) llmk_gelu_backward_inplace(dinp, pre_gelu, M * C, stream);
+    }
+
+    // (3) dW[OC,C] += dout^T . inp   (A(m=oc,k=row) stored [k][m], B(n=c,k=row) stored [k][n])
+    {
+        GemmArgs g{};
+        g.A = (const floatX*)dout; g.B = (const floatX*)inp; g.C = (floatX*)dweight;
+        g.M = OC; g.N = C; g.K = M; g.lda = OC; g.ldb = C; g.ldc = C;
+        const size_t tiles_big = (size_t)CEIL_DIV(OC, BIG_TILE) * CEIL_DIV(C, BIG_TILE);
+        const size_t tiles_small = (size_t)CEIL_DIV(OC, SMALL_TILE) * CEIL_DIV(C, SMALL_TILE);
+        const bool big = tiles_big >= 8;                          // split-K fills the machine when there are few big tiles
+        const size_t tiles = big ? tiles_big : tiles_small;
+        int splits = (int)max((size_t)1, (size_t)num_cu / tiles);
+        const int ksteps = CEIL_DIV(M, K_STEP);
+        splits = min(splits, max(1, ksteps / 8));                 // at least 8 K steps per split
+        const int steps_per = CEIL_DIV(ksteps, splits);
+        splits = CEIL_DIV(ksteps, steps_per);
+        g.k_per_split = steps_per * K_STEP;
+        const double tn_bytes = ((double)M * OC + (double)M * C + 2.0 * OC * C) * sizeof(floatX);
+        if (splits == 1) {
+            llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
+            launch_gemm<true, true, EPI_ACCUM>(g, 1, big, st);
+        } else {
+            const size_t mn = (size_t)OC * C;
+            g.partial = (float*)llmk::workspace(mn * splits * sizeof(float));
+            {
+                llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
+                launch_gemm<true, true, EPI_PARTIAL>(g, splits, big, st);
+            }
+            llmk::ProfScope prof("splitk_reduce", 0, (double)mn * splits * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
+            splitk_reduce_kernel<true><<<(unsigned)CEIL_DIV(mn / 4, (size_t)256), 256, 0, st>>>((floatX*)dweight, g.partial, mn, splits);
+            LAUNCH_CHECK();
+        }
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,366 @@
+// LayerNorm forward / fused residual+LayerNorm / residual add / LayerNorm backward for gfx950.
+//
+// All four are HBM-bound. Layout: one 64-lane wavefront owns one row at a time and keeps it in
+// registers (16-byte vectors, lane-interleaved so every load instruction of the wave covers a
+// contiguous 1 KiB), so each activation byte crosses HBM exactly once; weight/bias vectors of
+// the lane's columns stay in registers while the wave walks over its rows.
+//
+// Arithmetic follows the reference's CPU definitions: two-pass mean / biased variance with
+// eps 1e-5 (train_gpt2.c:78-118), backward per train_gpt2.c:120-161, statistics in fp32,
+// and — in the fused kernel — statistics of the residual AFTER rounding it to the storage
+// type (llmc/layernorm.cuh:178-184).
+#include "common.hpp"
+#include "../../include/llmk.h"
+
+namespace {
+
+constexpr int LN_BLOCK = 256;                 // 4 wavefronts per workgroup
+constexpr int LN_WAVES = LN_BLOCK / WAVE;
+constexpr int VN = vecX::N;
+
+// ---- forward ------------------------------------------------------------------------------
+// NV = vectors per lane (ceil(C / (VN*64))). RES: out-of-place residual add first.
+template <int NV, bool RES>
+__global__ void __launch_bounds__(LN_BLOCK)
+ln_forward_kernel(floatX* __restrict__ normed, floatX* __restrict__ residual, float* __restrict__ mean,
+                  float* __restrict__ rstd, const floatX* __restrict__ inp1, const floatX* __restrict__ inp2,
+                  const floatX* __restrict__ weight, const floatX* __restrict__ bias, int N, int C) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * LN_WAVES + (threadIdx.x >> 6);
+    const int nwaves = gridDim.x * LN_WAVES;
+    const int nvec = C / VN;
+
+    vecX w[NV], b[NV];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        int v = lane + i * 64;
+        if (v < nvec) { w[i] = ld_vec(weight + (size_t)v * VN); b[i] = ld_vec(bias + (size_t)v * VN); }
+    }
+    const float invC = 1.0f / (float)C;
+
+    for (int row = wave; row < N; row += nwaves) {
+        const size_t base = (size_t)row * C;
+        vecX x[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+                x[i] = ld_vec_nt(inp1 + base + (size_t)v * VN);
+                if (RES) {
+                    vecX y = ld_vec_nt(inp2 + base + (size_t)v * VN);
+#pragma unroll
+                    for (int k = 0; k < VN; k++) x[i][k] = from_f32<floatX>(to_f32(x[i][k]) + to_f32(y[k]));
+                    st_vec(residual + base + (size_t)v * VN, x[i]);
+                }
+            }
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; i++)
+            if (lane + i * 64 < nvec) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) s += to_f32(x[i][k]);
+            }
+        const float m = wave_sum(s) * invC;
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; i++)
+            if (lane + i * 64 < nvec) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) { float d = to_f32(x[i][k]) - m; q += d * d; }
+            }
+        const float var = wave_sum(q) * invC;
+        const float r = 1.0f / sqrtf(var + 1e-5f);
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+                vecX o;
+#pragma unroll
+                for (int k = 0; k < VN; k++)
+                    o[k] = from_f32<floatX>(r * (to_f32(x[i][k]) - m) * to_f32(w[i][k]) + to_f32(b[i][k]));
+                st_vec(normed + base + (size_t)v * VN, o);
+            }
+        }
+        if (lane == 0) {
+            if (mean) mean[row] = m;
+            if (rstd) rstd[row] = r;
+        }
+    }
+}
+
+// Any C (multiple of VN) beyond what fits in registers: re-reads the row (it sits in L2).
+template <bool RES>
+__global__ void __launch_bounds__(LN_BLOCK)
+ln_forward_generic_kernel(floatX* __restrict__ normed, floatX* __restrict__ residual, float* __restrict__ mean,
+                          float* __restrict__ rstd, const floatX* __restrict__ inp1,
+                          const floatX* __restrict__ inp2, const floatX* __restrict__ weight,
+                          const floatX* __restrict__ bias, int N, int C) {
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * LN_WAVES + (threadIdx.x >> 6);
+    const int nwaves = gridDim.x * LN_WAVES;
+    const int nvec = C / VN;
+    const float invC = 1.0f / (float)C;
+    for (int row = wave; row < N; row += nwaves) {
+        const size_t base = (size_t)row * C;
+        const floatX* src = inp1 + base;
+        if (RES) {
+            for (int v = lane; v < nvec; v += 64) {
+                vecX a = ld_vec(inp1 + base + (size_t)v * VN), y = ld_vec(inp2 + base + (size_t)v * VN);
+#pragma unroll
+                for (int k = 0; k < VN; k++) a[k] = from_f32<floatX>(to_f32(a[k]) + to_f32(y[k]));
+                st_vec(residual + base + (size_t)v * VN, a);
+            }
+            __threadfence_block();
+            src = residual + base;
+        }
+        float s = 0.f;
+        for (int v = lane; v < nvec; v += 64) {
+            vecX a = ld_vec(src + (size_t)v * VN);
+#pragma unroll
+            for (int k = 0; k < VN; k++) s += to_f32(a[k]);
+        }
+        const float m = wave_sum(s) * invC;
+        float q = 0.f;
+        for (int v = lane; v < nvec; v += 64) {
+            vecX a = ld_vec(src + (size_t)v * VN);
+#pragma unroll
+            for (int k = 0; k < VN; k++) { float d = to_f32(a[k]) - m; q += d * d; }
+        }
+        const float r = 1.0f / sqrtf(wave_sum(q) * invC + 1e-5f);
+        for (int v = lane; v < nvec; v += 64) {
+            vecX a = ld_vec(src + (size_t)v * VN), w = ld_vec(weight + (size_t)v * VN), b = ld_vec(bias + (size_t)v * VN), o;
+#pragma unroll
+            for (int k = 0; k < VN; k++) o[k] = from_f32<floatX>(r * (to_f32(a[k]) - m) * to_f32(w[k]) + to_f32(b[k]));
+            st_vec(normed + base + (size_t)v * VN, o);
+        }
+        if (lane == 0) {
+            if (mean) mean[row] = m;
+            if (rstd) rstd[row] = r;
+        }
+    }
+}
+
+template <bool RES>
+void launch_ln_forward(floatX* normed, floatX* residual, float* mean, float* rstd, const floatX* inp1,
+                       const floatX* inp2, const floatX* weight, const floatX* bias, int N, int C, hipStream_t st) {
+    const int nvec = C / VN;
+    const int nv = CEIL_DIV(nvec, 64);
+    const llmk::DeviceInfo& d = llmk::device_info();
+    int blocks = d.num_cu * 8;                       // 32 waves per CU, each walking ~N/(8192) rows
+    blocks = min(blocks, CEIL_DIV(N, LN_WAVES));
+    if (blocks < 1) blocks = 1;
+    const double bytes = (RES ? 4.0 : 2.0) * N * C * sizeof(floatX) + 2.0 * N * sizeof(float);
+    llmk::ProfScope prof(RES ? "fused_residual_forward" : "layernorm_forward", 0, bytes, st);
+#define LN_CASE(K)                                                                                            \
+    case K:                                                                                                   \
+        ln_forward_kernel<K, RES><<<blocks, LN_BLOCK, 0, st>>>(normed, residual, mean, rstd, inp1, inp2,      \
+                                                               weight, bias, N, C);                           \
+        break;
+    switch (nv) {
+        LN_CASE(1) LN_CASE(2) LN_CASE(3) LN_CASE(4) LN_CASE(5) LN_CASE(6) LN_CASE(7) LN_CASE(8)
+        default:
+            ln_forward_generic_kernel<RES><<<blocks, LN_BLOCK, 0, st>>>(normed, residual, mean, rstd, inp1, inp2,
+                                                                        weight, bias, N, C);
+    }
+#undef LN_CASE
+    LAUNCH_CHECK();
+}
+
+// ---- residual add --------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+residual_kernel(floatX* __restrict__ out, const floatX* __restrict__ a, const floatX* __restrict__ b, size_t nvec) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= nvec) return;
+    vecX x = ld_vec_nt(a + i * VN), y = ld_vec_nt(b + i * VN), o;
+#pragma unroll
+    for (int k = 0; k < VN; k++) o[k] = from_f32<floatX>(to_f32(x[k]) + to_f32(y[k]));
+    st_vec(out + i * VN, o);
+}
+
+// ---- backward ------------------------------------------------------------------------------
+// Each wave walks rows; per-lane fp32 accumulators hold dweight/dbias of the lane's columns.
+// At the end the 4 waves of a workgroup are added in wave order through LDS and the workgroup's
+// partial goes to scratch[block][2][C]; a second kernel adds the partials in block order, so
+// the result does not depend on scheduling (no atomics).
+template <int NV>
+__global__ void __launch_bounds__(LN_BLOCK)
+ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
+                   const floatX* __restrict__ inp, const floatX* __restrict__ weight,
+                   const float* __restrict__ mean, const float* __restrict__ rstd, int N, int C) {
+    extern __shared__ float lds[];   // [LN_WAVES-1][2][C]
+    const int lane = threadIdx.x & 63;
+    const int wid = threadIdx.x >> 6;
+    const int wave = blockIdx.x * LN_WAVES + wid;
+    const int nwaves = gridDim.x * LN_WAVES;
+    const int nvec = C / VN;
+    const float invC = 1.0f / (float)C;
+
+    float w[NV][VN], dw[NV][VN], db[NV][VN];
+#pragma unroll
+    for (int i = 0; i < NV; i++) {
+        int v = lane + i * 64;
+        vecX wv;
+        if (v < nvec) wv = ld_vec(weight + (size_t)v * VN);
+#pragma unroll
+        for (int k = 0; k < VN; k++) { w[i][k] = v < nvec ? to_f32(wv[k]) : 0.f; dw[i][k] = 0.f; db[i][k] = 0.f; }
+    }
+
+    for (int row = wave; row < N; row += nwaves) {
+        const size_t base = (size_t)row * C;
+        vecX g[NV], x[NV], di[NV];
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+                g[i] = ld_vec_nt(dout + base + (size_t)v * VN);
+                x[i] = ld_vec_nt(inp + base + (size_t)v * VN);
+                di[i] = ld_vec(dinp + base + (size_t)v * VN);
+            }
+        }
+        const float m = mean[row], r = rstd[row];
+        float a = 0.f, bsum = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; i++)
+            if (lane + i * 64 < nvec) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) {
+                    float nh = (to_f32(x[i][k]) - m) * r, dn = w[i][k] * to_f32(g[i][k]);
+                    a += dn;
+                    bsum += dn * nh;
+                }
+            }
+        a = wave_sum(a) * invC;
+        bsum = wave_sum(bsum) * invC;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+                vecX o;
+#pragma unroll
+                for (int k = 0; k < VN; k++) {
+                    float gk = to_f32(g[i][k]);
+                    float nh = (to_f32(x[i][k]) - m) * r, dn = w[i][k] * gk;
+                    db[i][k] += gk;
+                    dw[i][k] += nh * gk;
+                    o[k] = from_f32<floatX>(to_f32(di[i][k]) + (dn - a - nh * bsum) * r);
+                }
+                st_vec(dinp + base + (size_t)v * VN, o);
+            }
+        }
+    }
+
+    // workgroup reduction in fixed wave order
+    if (wid > 0) {
+        float* dst = lds + (size_t)(wid - 1) * 2 * C;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) { dst[v * VN + k] = dw[i][k]; dst[C + v * VN + k] = db[i][k]; }
+            }
+        }
+    }
+    __syncthreads();
+    if (wid == 0) {
+        float* out = partial + (size_t)blockIdx.x * 2 * C;
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            int v = lane + i * 64;
+            if (v < nvec) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) {
+                    float sw = dw[i][k], sb = db[i][k];
+                    for (int o = 0; o < LN_WAVES - 1; o++) {
+                        sw += lds[(size_t)o * 2 * C + v * VN + k];
+                        sb += lds[(size_t)o * 2 * C + C + v * VN + k];
+                    }
+                    out[v * VN + k] = sw;
+                    out[C + v * VN + k] = sb;
+                }
+            }
+        }
+    }
+}
+
+// dweight[c] += sum_blocks partial[b][0][c]; dbias likewise. One thread per column.
+__global__ void __launch_bounds__(256)
+ln_backward_reduce_kernel(floatX* __restrict__ dweight, floatX* __restrict__ dbias, const float* __restrict__ partial,
+                          int nblocks, int C) {
+    int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= 2 * C) return;
+    float s = 0.f;
+    for (int b = 0; b < nblocks; b++) s += partial[(size_t)b * 2 * C + c];
+    floatX* dst = c < C ? dweight + c : dbias + (c - C);
+    *dst = from_f32<floatX>(to_f32(*dst) + s);
+}
+
+int ln_backward_blocks() { return llmk::device_info().num_cu * 4; }
+
+}  // namespace
+
+extern "C" {
+
+void llmk_layernorm_forward(void* out, float* mean, float* rstd, const void* inp, const void* weight,
+                            const void* bias, int B, int T, int C, void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(C > 0 && C % VN == 0, "layernorm_forward: C=%d must be a multiple of %d", C, VN);
+    if ((size_t)B * T == 0) return;
+    launch_ln_forward<false>((floatX*)out, nullptr, mean, rstd, (const floatX*)inp, nullptr, (const floatX*)weight,
+                             (const floatX*)bias, B * T, C, (hipStream_t)stream);
+}
+
+void llmk_fused_residual_forward5(void* residual, void* normed, float* mean, float* rstd, const void* inp1,
+                                  const void* inp2, const void* weight, const void* bias, int N, int C,
+                                  void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(C > 0 && C % VN == 0, "fused_residual_forward5: C=%d must be a multiple of %d", C, VN);
+    if (N == 0) return;
+    launch_ln_forward<true>((floatX*)normed, (floatX*)residual, mean, rstd, (const floatX*)inp1, (const floatX*)inp2,
+                            (const floatX*)weight, (const floatX*)bias, N, C, (hipStream_t)stream);
+}
+
+void llmk_residual_forward(void* out, const void* inp1, const void* inp2, int N, void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(N % VN == 0, "residual_forward: N=%d must be a multiple of %d", N, VN);
+    if (N == 0) return;
+    size_t nvec = (size_t)N / VN;
+    llmk::ProfScope prof("residual_forward", 0, 3.0 * N * sizeof(floatX), (hipStream_t)stream);
+    residual_kernel<<<(unsigned)CEIL_DIV(nvec, (size_t)256), 256, 0, (hipStream_t)stream>>>(
+        (floatX*)out, (const floatX*)inp1, (const floatX*)inp2, nvec);
+    LAUNCH_CHECK();
+}
+
+size_t llmk_layernorm_backward_scratch_floats(int C) { return (size_t)ln_backward_blocks() * 2 * C; }
+
+void llmk_layernorm_backward(void* dinp, void* dweight, void* dbias, float* scratch, const void* dout,
+                             const void* inp, const void* weight, const float* mean, const float* rstd, int B,
+                             int T, int C, void* stream) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(C > 0 && C % VN == 0, "layernorm_backward: C=%d must be a multiple of %d", C, VN);
+    const int nv = CEIL_DIV(C / VN, 64);
+    LLMK_REQUIRE(nv <= 8, "layernorm_backward: C=%d too large (max %d)", C, 8 * 64 * VN);
+    const int N = B * T;
+    if (N == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    int blocks = min(ln_backward_blocks(), CEIL_DIV(N, LN_WAVES));
+    size_t smem = (size_t)(LN_WAVES - 1) * 2 * C * sizeof(float);
+    {
+    llmk::ProfScope prof("layernorm_backward", 0, 4.0 * N * C * sizeof(floatX) + 2.0 * N * sizeof(float), st);
+#define LNB_CASE(K)                                                                                          \
+    case K:                                                                                                  \
+        ln_backward_kernel<K><<<blocks, LN_BLOCK, smem, st>>>((floatX*)dinp, scratch, (const floatX*)dout,   \
+                                                              (const floatX*)inp, (const floatX*)weight,    \
+                                                              mean, rstd, N, C);                             \
+        break;
+    switch (nv) { LNB_CASE(1) LNB_CASE(2) LNB_CASE(3) LNB_CASE(4) LNB_CASE(5) LNB_CASE(6) LNB_CASE(7) LNB_CASE(8) }
+#undef LNB_CASE
+    LAUNCH_CHECK();
+    }
+    llmk::ProfScope prof2("layernorm_backward_reduce", 0, (double)blocks * 2 * C * sizeof(float), st);
+    ln_backward_reduce_kernel<<<CEIL_DIV(2 * C, 256), 256, 0, st>>>((floatX*)dweight, (floatX*)dbias, scratch, blocks, C);
+    LAUNCH_CHECK();
+}
+
+}  // extern "C"

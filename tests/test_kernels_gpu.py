@@ -1,0 +1,461 @@
+"""Per-kernel parity: every entry point of include/llmk.h, called through the C ABI on the GPU,
+against the CPU oracle (oracle/cpu_ref.c) on the same seeded inputs.
+
+fp32 library: tolerances of the reference's own kernel harness (dev/cuda/*.cu, 1e-5 .. 1e-3).
+bf16 library: the oracle is fed the bf16-rounded inputs; outputs may differ by bf16 rounding of the
+result (relative 2^-8) plus fp32 accumulation-order noise.
+"""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import gpu_lib as G
+import oracle_lib as ol
+
+pytestmark = pytest.mark.gpu
+
+PRECS = ["fp32", "bf16"]
+
+
+def rnd(shape, seed, scale=1.0):
+    return (np.random.RandomState(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def tol(precision, fp32_atol, bf16_rel=1.0 / 128, bf16_atol=None):
+    if precision == "fp32":
+        return dict(rtol=1e-5, atol=fp32_atol)
+    return dict(rtol=bf16_rel, atol=bf16_atol if bf16_atol is not None else fp32_atol)
+
+
+def close(actual, desired, rtol, atol, what=""):
+    np.testing.assert_allclose(actual, desired, rtol=rtol, atol=atol, err_msg=what)
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _cuda():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    yield
+    torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("B,T,C,V", [(2, 8, 64, 100), (4, 64, 768, 50257)])
+def test_encoder_forward(precision, B, T, C, V):
+    L = G.lib(precision)
+    wte, wpe = G.rounded(rnd((V, C), 0), precision), G.rounded(rnd((T, C), 1), precision)
+    inp = np.random.RandomState(2).randint(0, V, B * T).astype(np.int32)
+    ref = np.zeros((B, T, C), np.float32)
+    ol.cref().cref_encoder_forward(ref, inp, wte, wpe, B, T, C)
+    d_out = G.dev(np.zeros((B, T, C), np.float32), precision)
+    d_wte, d_wpe, d_inp = G.dev(wte, precision), G.dev(wpe, precision), G.dev(inp)
+    L.llmk_encoder_forward(G.ptr(d_out), G.ptr(d_inp), G.ptr(d_wte), G.ptr(d_wpe), B, T, C, None)
+    close(G.host(d_out), ref, **tol(precision, 1e-6, bf16_atol=1e-2))
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("B,T,C,V", [(2, 16, 64, 20), (8, 256, 768, 300), (3, 32, 1600, 50)])
+def test_encoder_backward(precision, B, T, C, V):
+    L = G.lib(precision)
+    N = B * T
+    rs = np.random.RandomState(3)
+    inp = rs.randint(0, V, N).astype(np.int32)
+    inp[rs.rand(N) < 0.3] = 7                       # one very frequent token: long bucket, all four waves busy
+    dout = G.rounded(rnd((B, T, C), 4), precision)
+    dwte0, dwpe0 = G.rounded(rnd((V, C), 5), precision), G.rounded(rnd((T, C), 6), precision)
+    rwte, rwpe = dwte0.copy(), dwpe0.copy()
+    ol.cref().cref_encoder_backward(rwte, rwpe, dout, inp, B, T, C)
+    vn = 8 if precision == "bf16" else 4
+    ncg = -(-C // (64 * vn))
+    import torch
+    scratch = torch.zeros(N * ncg * 20 + 64, dtype=torch.uint8, device="cuda")
+    wl = np.zeros(N * ncg, np.int32); bk = np.zeros(4 * N * ncg, np.int32)
+    d_wte, d_wpe, d_dout, d_inp = G.dev(dwte0, precision), G.dev(dwpe0, precision), G.dev(dout, precision), G.dev(inp)
+    L.llmk_encoder_backward(G.ptr(d_wte), G.ptr(d_wpe), G.ptr(scratch), wl.ctypes.data_as(C.c_void_p),
+                            bk.ctypes.data_as(C.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(C.c_void_p),
+                            B, T, C, 1234, None)
+    # stochastic rounding lands on one of the two bf16 neighbours of the exact sum: 1 ulp = 2^-7 relative
+    close(G.host(d_wte), rwte, **tol(precision, 1e-4, bf16_rel=1.0 / 64, bf16_atol=2e-2), what="dwte")
+    close(G.host(d_wpe), rwpe, **tol(precision, 1e-4, bf16_rel=1.0 / 64, bf16_atol=2e-2), what="dwpe")
+    # determinism: same call, same bits
+    d_wte2, d_wpe2 = G.dev(dwte0, precision), G.dev(dwpe0, precision)
+    L.llmk_encoder_backward(G.ptr(d_wte2), G.ptr(d_wpe2), G.ptr(scratch), wl.ctypes.data_as(C.c_void_p),
+                            bk.ctypes.data_as(C.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(C.c_void_p),
+                            B, T, C, 1234, None)
+    G.sync()
+    assert torch.equal(d_wte, d_wte2) and torch.equal(d_wpe, d_wpe2)
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("N,C", [(7, 64), (1024, 768), (300, 1600), (16, 4104)])
+def test_layernorm_forward_and_fused_residual(precision, N, C):
+    L = G.lib(precision)
+    x, y = G.rounded(rnd((N, C), 0, 2.0) + 0.5, precision), G.rounded(rnd((N, C), 1), precision)
+    w, b = G.rounded(rnd(C, 2), precision), G.rounded(rnd(C, 3), precision)
+    ro = np.zeros((N, C), np.float32); rm = np.zeros(N, np.float32); rr = np.zeros(N, np.float32)
+    ol.cref().cref_layernorm_forward(ro, rm.ctypes.data, rr.ctypes.data, x, w, b, N, C)
+    d_o = G.dev(np.zeros((N, C), np.float32), precision)
+    d_m, d_r = G.dev(np.zeros(N, np.float32)), G.dev(np.zeros(N, np.float32))
+    d_x, d_y, d_w, d_b = (G.dev(a, precision) for a in (x, y, w, b))
+    L.llmk_layernorm_forward(G.ptr(d_o), G.ptr(d_m), G.ptr(d_r), G.ptr(d_x), G.ptr(d_w), G.ptr(d_b), 1, N, C, None)
+    close(G.host(d_m), rm, rtol=1e-5, atol=1e-5, what="mean")
+    close(G.host(d_r), rr, rtol=2e-5, atol=1e-6, what="rstd")
+    close(G.host(d_o), ro, **tol(precision, 2e-5, bf16_atol=2e-2), what="out")      # dev/cuda/layernorm_forward.cu:590
+    # mean/rstd are optional
+    d_o2 = G.dev(np.zeros((N, C), np.float32), precision)
+    L.llmk_layernorm_forward(G.ptr(d_o2), None, None, G.ptr(d_x), G.ptr(d_w), G.ptr(d_b), 1, N, C, None)
+    import torch
+    G.sync()
+    assert torch.equal(d_o, d_o2)
+    # fused residual: residual = round(x + y), statistics of the rounded sum
+    res = G.rounded(x + y, precision)
+    ol.cref().cref_layernorm_forward(ro, rm.ctypes.data, rr.ctypes.data, res, w, b, N, C)
+    d_res = G.dev(np.zeros((N, C), np.float32), precision)
+    L.llmk_fused_residual_forward5(G.ptr(d_res), G.ptr(d_o), G.ptr(d_m), G.ptr(d_r), G.ptr(d_x), G.ptr(d_y), G.ptr(d_w),
+                                   G.ptr(d_b), N, C, None)
+    np.testing.assert_array_equal(G.host(d_res), res)
+    close(G.host(d_m), rm, rtol=1e-5, atol=1e-5)
+    close(G.host(d_o), ro, **tol(precision, 2e-5, bf16_atol=2e-2))
+    # plain residual add
+    d_sum = G.dev(np.zeros((N, C), np.float32), precision)
+    L.llmk_residual_forward(G.ptr(d_sum), G.ptr(d_x), G.ptr(d_y), N * C, None)
+    np.testing.assert_array_equal(G.host(d_sum), res)
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("N,C", [(9, 64), (2048, 768), (520, 1600)])
+def test_layernorm_backward(precision, N, C):
+    L = G.lib(precision)
+    x, g = G.rounded(rnd((N, C), 0, 1.5), precision), G.rounded(rnd((N, C), 1), precision)
+    w = G.rounded(rnd(C, 2), precision)
+    rm = np.zeros(N, np.float32); rr = np.zeros(N, np.float32); tmp = np.zeros((N, C), np.float32)
+    ol.cref().cref_layernorm_forward(tmp, rm.ctypes.data, rr.ctypes.data, x, w, np.zeros(C, np.float32), N, C)
+    dx0, dw0, db0 = G.rounded(rnd((N, C), 3), precision), G.rounded(rnd(C, 4), precision), G.rounded(rnd(C, 5), precision)
+    rdx, rdw, rdb = dx0.copy(), dw0.copy(), db0.copy()
+    ol.cref().cref_layernorm_backward(rdx, rdw, rdb, g, x, w, rm, rr, N, C)
+    d_dx, d_dw, d_db = G.dev(dx0, precision), G.dev(dw0, precision), G.dev(db0, precision)
+    d_g, d_x, d_w = G.dev(g, precision), G.dev(x, precision), G.dev(w, precision)
+    d_m, d_r = G.dev(rm), G.dev(rr)
+    import torch
+    scratch = torch.empty(L.llmk_layernorm_backward_scratch_floats(C), dtype=torch.float32, device="cuda")
+    L.llmk_layernorm_backward(G.ptr(d_dx), G.ptr(d_dw), G.ptr(d_db), G.ptr(scratch), G.ptr(d_g), G.ptr(d_x), G.ptr(d_w),
+                              G.ptr(d_m), G.ptr(d_r), 1, N, C, None)
+    # dev/cuda/layernorm_backward.cu:1506-1507: dinp 1e-3 / 1e-1, dweight/dbias 1e-3 / 5e-1
+    close(G.host(d_dx), rdx, **tol(precision, 1e-4, bf16_atol=5e-2), what="dinp")
+    s = np.sqrt(N)
+    close(G.host(d_dw), rdw, **tol(precision, 1e-4 * s, bf16_rel=1.0 / 64, bf16_atol=1e-2 * s), what="dweight")
+    close(G.host(d_db), rdb, **tol(precision, 1e-4 * s, bf16_rel=1.0 / 64, bf16_atol=1e-2 * s), what="dbias")
+    G.check_no_error(L)
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+def test_gelu(precision):
+    L = G.lib(precision)
+    n = 8 * 1024 + 64
+    x = G.rounded(np.concatenate([rnd(n - 8, 0, 3.0), np.array([0, -0.0, 20, -20, 1e-3, 5, -5, 0.5], np.float32)]), precision)
+    g = G.rounded(rnd(n, 1), precision)
+    ro = np.zeros(n, np.float32); ol.cref().cref_gelu_forward(ro, x, n)
+    d_x, d_o = G.dev(x, precision), G.dev(np.zeros(n, np.float32), precision)
+    L.llmk_gelu_forward(G.ptr(d_o), G.ptr(d_x), n, None)
+    close(G.host(d_o), ro, **tol(precision, 1e-5, bf16_atol=1e-2))                # dev/cuda/gelu_forward.cu
+    rd = np.zeros(n, np.float32); ol.cref().cref_gelu_backward(rd, x, g, n)
+    d_g = G.dev(g, precision)
+    L.llmk_gelu_backward_inplace(G.ptr(d_g), G.ptr(d_x), n, None)
+    close(G.host(d_g), rd, **tol(precision, 1e-5, bf16_atol=1e-2))
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("N,V,P", [(5, 100, 128), (64, 50257, 50304), (3, 8003, 8064), (2, 130000, 130048)])
+def test_fused_classifier(precision, N, V, P):
+    L = G.lib(precision)
+    z = rnd((N, P), 0, 2.0)
+    rs = np.random.RandomState(1)
+    for r in range(N):                                   # a few outliers per row (dev/cuda/classifier_fused.cu:689-696)
+        z[r, rs.randint(0, V, 3)] *= 20
+    z = G.rounded(z, precision)
+    tg = rs.randint(0, V, N).astype(np.int32); tg[0] = V - 1
+    probs = np.zeros((N, P), np.float32); rl = np.zeros(N, np.float32)
+    ol.cref().cref_softmax_crossentropy_forward(probs, rl.ctypes.data, z, tg.ctypes.data, N, V, P)
+    dloss = 1.0 / N
+    rd = np.zeros((N, P), np.float32)
+    ol.cref().cref_crossentropy_softmax_backward(rd, probs, tg, dloss, N, V, P)
+    rd[:, V:] = z[:, V:]                                  # padded columns keep their logit values
+    base = rnd(N, 5)
+    d_z, d_l, d_t = G.dev(z, precision), G.dev(base.copy()), G.dev(tg)
+    # losses only
+    L.llmk_fused_classifier(G.ptr(d_z), G.ptr(d_l), dloss, G.ptr(d_t), 1, N, V, P, 0, None)
+    close(G.host(d_l), base + rl, rtol=1e-5, atol=1e-4, what="losses accumulate")
+    np.testing.assert_array_equal(G.host(d_z), z)
+    # losses + dlogits in place
+    d_l = G.dev(np.zeros(N, np.float32))
+    L.llmk_fused_classifier(G.ptr(d_z), G.ptr(d_l), dloss, G.ptr(d_t), 1, N, V, P, 1, None)
+    close(G.host(d_l), rl, rtol=1e-5, atol=1e-4)                                  # classifier_fused.cu:739
+    out = G.host(d_z)
+    close(out[:, :V], rd[:, :V], **tol(precision, 1e-6, bf16_rel=1.0 / 64, bf16_atol=1e-5), what="dlogits")
+    np.testing.assert_array_equal(out[:, V:], z[:, V:])
+    G.check_no_error(L)
+
+
+# ------------------------------------------------------------------------------------------------
+def run_matmul_forward(L, precision, x, w, b, pre_gelu, fusion):
+    M, Cc = x.shape
+    OC = w.shape[0]
+    d_x, d_w = G.dev(x, precision), G.dev(w, precision)
+    d_b = G.dev(b, precision) if b is not None else None
+    d_o = G.dev(np.zeros((M, OC), np.float32), precision)
+    d_pre = G.dev(np.zeros((M, OC), np.float32), precision) if pre_gelu else None
+    L.llmk_matmul_forward(G.ptr(d_o), G.ptr(d_x), G.ptr(d_w), G.ptr(d_b), 1, M, Cc, OC, None, G.ptr(d_pre), fusion)
+    return G.host(d_o), (G.host(d_pre) if pre_gelu else None)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("M,Cc,OC,bias", [(64, 64, 64, True), (200, 72, 136, True), (256, 768, 2304, True),
+                                           (512, 3072, 768, True), (128, 768, 50304, False),
+                                           (4096, 256, 4096, True), (4100, 192, 4360, False)])
+def test_matmul_forward(precision, M, Cc, OC, bias):
+    L = G.lib(precision)
+    x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
+    b = G.rounded(rnd(OC, 2), precision) if bias else None
+    ref = x.astype(np.float64) @ w.astype(np.float64).T + (b if bias else 0)
+    if M * Cc * OC <= 256 * 768 * 2304:                  # the oracle's loops, where they finish quickly
+        r2 = np.zeros((M, OC), np.float32)
+        ol.cref().cref_matmul_forward(r2, x, w, b.ctypes.data if bias else None, M, Cc, OC)
+        close(r2, ref, rtol=1e-4, atol=1e-4)
+    out, _ = run_matmul_forward(L, precision, x, w, b, False, 1)
+    sc = np.sqrt(Cc) * 0.1
+    close(out, ref, **tol(precision, 2e-5 * sc, bf16_atol=1e-2 * sc))
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("fusion", [0, 1])
+@pytest.mark.parametrize("M,Cc,OC", [(192, 128, 512), (4096, 128, 4096)])
+def test_matmul_forward_gelu(precision, fusion, M, Cc, OC):
+    L = G.lib(precision)
+    x, w, b = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision), G.rounded(rnd(OC, 2), precision)
+    pre = (x.astype(np.float64) @ w.astype(np.float64).T + b).astype(np.float32)
+    out, got_pre = run_matmul_forward(L, precision, x, w, b, True, fusion)
+    close(got_pre, pre, **tol(precision, 5e-5, bf16_atol=2e-2), what="pre_gelu")
+    ref = np.zeros_like(got_pre)
+    ol.cref().cref_gelu_forward(ref.reshape(-1), np.ascontiguousarray(got_pre).reshape(-1), got_pre.size)
+    close(out, ref, **tol(precision, 1e-5, bf16_atol=1e-2), what="gelu(pre_gelu)")
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("M,Cc,OC,bias", [(64, 64, 64, True), (200, 72, 136, True), (256, 768, 2304, True),
+                                           (1024, 3072, 768, True), (8192, 768, 768, True), (4096, 2048, 2048, False),
+                                           (128, 256, 50304, False)])
+def test_matmul_backward(precision, M, Cc, OC, bias):
+    L = G.lib(precision)
+    x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
+    g = G.rounded(rnd((M, OC), 2), precision)
+    dw0, db0 = G.rounded(rnd((OC, Cc), 3), precision), G.rounded(rnd(OC, 4), precision)
+    g64 = g.astype(np.float64)
+    r_dx = g64 @ w.astype(np.float64)
+    r_dw = dw0 + g64.T @ x.astype(np.float64)
+    r_db = db0 + g64.sum(0)
+    if M * Cc * OC <= 256 * 768 * 2304:
+        c_dx = np.zeros((M, Cc), np.float32); c_dw = dw0.copy(); c_db = db0.copy()
+        ol.cref().cref_matmul_backward(c_dx.ctypes.data, c_dw, c_db.ctypes.data, g, x, w, M, Cc, OC)
+        close(c_dx, r_dx, rtol=1e-4, atol=1e-3); close(c_dw, r_dw, rtol=1e-4, atol=1e-3); close(c_db, r_db, rtol=1e-4, atol=1e-3)
+    import torch
+    d_dx = G.dev(np.full((M, Cc), 7.0, np.float32), precision)        # dinp is overwritten, not accumulated
+    d_dw, d_db = G.dev(dw0, precision), (G.dev(db0, precision) if bias else None)
+    d_g, d_x, d_w = G.dev(g, precision), G.dev(x, precision), G.dev(w, precision)
+    scratch = torch.empty(max(1, L.llmk_matmul_backward_bias_scratch_floats(OC)), dtype=torch.float32, device="cuda")
+    L.llmk_matmul_backward(G.ptr(d_dx), G.ptr(d_dw), G.ptr(d_db), G.ptr(d_g), G.ptr(d_x), G.ptr(d_w), G.ptr(scratch),
+                           1, M, Cc, OC, None, None, 1)
+    close(G.host(d_dx), r_dx, **tol(precision, 3e-5 * np.sqrt(OC), bf16_atol=1e-3 * np.sqrt(OC)), what="dinp")
+    close(G.host(d_dw), r_dw, **tol(precision, 3e-5 * np.sqrt(M), bf16_atol=1e-2 * np.sqrt(M)), what="dweight")
+    if bias:
+        close(G.host(d_db), r_db, **tol(precision, 3e-5 * np.sqrt(M), bf16_atol=1e-2 * np.sqrt(M)), what="dbias")
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("fusion", [0, 2])
+def test_matmul_backward_gelu(precision, fusion):
+    L = G.lib(precision)
+    M, Cc, OC = 320, 512, 128           # dinp has the 4C width: (M, Cc) with pre_gelu of the same shape
+    x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
+    g, pre = G.rounded(rnd((M, OC), 2), precision), G.rounded(rnd((M, Cc), 3, 2.0), precision)
+    lin = G.rounded((g.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), precision)
+    ref = np.zeros((M, Cc), np.float32)
+    ol.cref().cref_gelu_backward(ref.reshape(-1), pre.reshape(-1), lin.reshape(-1), M * Cc)
+    import torch
+    d_dx, d_dw = G.dev(np.zeros((M, Cc), np.float32), precision), G.dev(np.zeros((OC, Cc), np.float32), precision)
+    d_g, d_x, d_w, d_pre = G.dev(g, precision), G.dev(x, precision), G.dev(w, precision), G.dev(pre, precision)
+    L.llmk_matmul_backward(G.ptr(d_dx), G.ptr(d_dw), None, G.ptr(d_g), G.ptr(d_x), G.ptr(d_w), None, 1, M, Cc, OC, None,
+                           G.ptr(d_pre), fusion)
+    close(G.host(d_dx), ref, **tol(precision, 1e-4, bf16_rel=1.0 / 32, bf16_atol=3e-2))
+    G.check_no_error(L)
+
+
+# ------------------------------------------------------------------------------------------------
+def attention_case(precision, B, T, NH, seed=0):
+    hs = 64
+    Cc = NH * hs
+    qkv = G.rounded(rnd((B, T, 3 * Cc), seed, 1.0), precision)
+    g = G.rounded(rnd((B, T, Cc), seed + 1), precision)
+    o = np.zeros((B, T, Cc), np.float32); lse = np.zeros((B, NH, T), np.float32)
+    ol.cref().cref_attention_forward(o, None, lse.ctypes.data, qkv, B, T, Cc, NH)
+    d = np.zeros((B, T, 3 * Cc), np.float32)
+    ol.cref().cref_attention_backward(d, g, qkv, None, B, T, Cc, NH)
+    return qkv, g, o, lse, d, Cc
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("B,T,NH", [(2, 64, 2), (1, 128, 3), (2, 200, 2), (1, 1, 2), (1, 1024, 2), (2, 384, 12)])
+def test_attention_forward_backward(precision, B, T, NH):
+    L = G.lib(precision)
+    qkv, g, ro, rlse, rd, Cc = attention_case(precision, B, T, NH)
+    d_qkv, d_g = G.dev(qkv, precision), G.dev(g, precision)
+    d_o = G.dev(np.zeros((B, T, Cc), np.float32), precision)
+    d_lse = G.dev(np.zeros((B, NH, T), np.float32))
+    L.llmk_attention_forward(G.ptr(d_o), G.ptr(d_lse), G.ptr(d_qkv), B, T, NH, Cc, None)
+    close(G.host(d_o), ro, **tol(precision, 1e-5, bf16_atol=2e-2), what="out")        # dev/cuda/attention_forward.cu:1330
+    close(G.host(d_lse), rlse, rtol=1e-5, atol=(1e-4 if precision == "fp32" else 2e-2), what="stats")
+    # inference mode: no statistics
+    d_o2 = G.dev(np.zeros((B, T, Cc), np.float32), precision)
+    L.llmk_attention_forward(G.ptr(d_o2), None, G.ptr(d_qkv), B, T, NH, Cc, None)
+    import torch
+    G.sync()
+    assert torch.equal(d_o, d_o2)
+    d_d = G.dev(np.full((B, T, 3 * Cc), 3.0, np.float32), precision)                  # overwritten, not accumulated
+    L.llmk_attention_backward(G.ptr(d_d), G.ptr(d_g), G.ptr(d_qkv), G.ptr(d_o), G.ptr(d_lse), B, T, NH, Cc, None)
+    scale = np.abs(rd).max()
+    close(G.host(d_d), rd, **tol(precision, 1e-4 * scale, bf16_rel=1.0 / 32, bf16_atol=2e-2 * scale), what="dqkv")
+    # causality at the kernel level: future tokens do not change earlier outputs
+    if T >= 64:
+        q2 = qkv.copy(); q2[:, T // 2:] += 1.0
+        d_q2 = G.dev(G.rounded(q2, precision), precision)
+        L.llmk_attention_forward(G.ptr(d_o2), None, G.ptr(d_q2), B, T, NH, Cc, None)
+        G.sync()
+        assert torch.equal(d_o[:, :T // 2], d_o2[:, :T // 2])
+    G.check_no_error(L)
+
+
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("use_master", [True, False])
+def test_adamw_update(precision, use_master):
+    L = G.lib(precision)
+    n, slices, stride = 5000 * 8, 3, 5000 * 8 + 64
+    tot = stride * slices
+    p0 = G.rounded(rnd(tot, 0, 0.05), precision); g = G.rounded(rnd(tot, 1, 0.01), precision)
+    m0, v0 = rnd(tot, 2, 0.01), np.abs(rnd(tot, 3, 1e-4))
+    master0 = p0 + rnd(tot, 4, 1e-4) if use_master else None
+    lr, b1, b2, t, eps, wd, gs, seed = 1e-3, 0.9, 0.95, 3, 1e-8, 0.1, 0.5, 42
+    rp, rm, rv = p0.copy(), m0.copy(), v0.copy()
+    rmaster = master0.copy() if use_master else None
+    for s in range(slices):
+        sl = slice(s * stride, s * stride + n)
+        mm, vv = rm[sl].copy(), rv[sl].copy()
+        ms = rmaster[sl].copy() if use_master else None
+        if precision == "bf16":
+            pb, gb = ol.to_bf16_bits(rp[sl]), ol.to_bf16_bits(g[sl])
+            ol.cref().cref_adamw_mixed(pb, ms.ctypes.data if use_master else None, gb, mm, vv, n, lr, b1, b2, t, eps, wd, gs, seed, s)
+            rp[sl] = ol.from_bf16_bits(pb)
+        else:
+            pp = rp[sl].copy()
+            ol.cref().cref_adamw_f32(pp, ms.ctypes.data if use_master else None, g[sl].copy(), mm, vv, n, lr, b1, b2, t, eps, wd, gs)
+            rp[sl] = pp
+        rm[sl], rv[sl] = mm, vv
+        if use_master:
+            rmaster[sl] = ms
+    d_p, d_g, d_m, d_v = G.dev(p0, precision), G.dev(g, precision), G.dev(m0), G.dev(v0)
+    d_ms = G.dev(master0) if use_master else None
+    L.llmk_adamw_update(G.ptr(d_p), G.ptr(d_ms), G.ptr(d_g), G.ptr(d_m), G.ptr(d_v), n, stride, stride, stride, slices,
+                        lr, b1, b2, t, eps, wd, gs, seed, None)
+    close(G.host(d_m), rm, rtol=1e-6, atol=1e-9, what="m")
+    close(G.host(d_v), rv, rtol=1e-6, atol=1e-12, what="v")
+    if use_master:
+        close(G.host(d_ms), rmaster, rtol=1e-6, atol=1e-8, what="master")
+    got = G.host(d_p)
+    if precision == "fp32":
+        close(got, rp, rtol=1e-6, atol=1e-8)
+    else:
+        # the low-precision parameter is the stochastic rounding of the fp32 result with the reference's noise word:
+        # bit-exact given the GPU's own fp32 value (master), and equal to the oracle's wherever the fp32 values agree
+        if use_master:
+            gm = G.host(d_ms)
+            for s in range(slices):
+                for i in list(range(0, 64)) + list(range(n - 64, n)) + list(np.random.RandomState(s).randint(0, n, 200)):
+                    k = s * stride + int(i)
+                    want = ol.cref().cref_stochastic_round_bf16(float(gm[k]), ol.cref().cref_adamw_noise(int(i), s, seed))
+                    assert ol.to_bf16_bits(got[k:k + 1])[0] == want, (s, i)
+        close(got, rp, rtol=1.0 / 128, atol=1e-6)
+        assert (got != rp).mean() < 1e-3
+    # gaps between slices untouched
+    for s in range(slices):
+        np.testing.assert_array_equal(got[s * stride + n:(s + 1) * stride], p0[s * stride + n:(s + 1) * stride])
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+def test_adamw_unaligned_tail_and_init_from_master(precision):
+    L = G.lib(precision)
+    n = 1003                                         # not a multiple of the vector width: scalar path
+    p0 = G.rounded(rnd(n, 0, 0.05), precision); g = G.rounded(rnd(n, 1, 0.01), precision)
+    d_p, d_g = G.dev(p0, precision), G.dev(g, precision)
+    d_m, d_v = G.dev(np.zeros(n, np.float32)), G.dev(np.zeros(n, np.float32))
+    d_ms = G.dev(np.zeros(n, np.float32))
+    L.llmk_copy_and_cast_to_f32(G.ptr(d_ms), G.ptr(d_p), n, 0, 0, 1, None)
+    np.testing.assert_array_equal(G.host(d_ms), p0)
+    L.llmk_adamw_update(G.ptr(d_p), G.ptr(d_ms), G.ptr(d_g), G.ptr(d_m), G.ptr(d_v), n, 0, 0, 0, 1,
+                        1e-2, 0.9, 0.999, 1, 1e-8, 0.0, 1.0, 7, None)
+    # first step from zero state is sign descent: p - lr * g/(|g|+eps)
+    want = p0 - 1e-2 * g / (np.abs(g) + 1e-8)
+    close(G.host(d_ms), want, rtol=1e-5, atol=1e-7)
+    # init_from_master reproduces exactly the parameters the update wrote (same seed => same rounding)
+    d_p2 = G.dev(np.zeros(n, np.float32), precision)
+    L.llmk_init_from_master(G.ptr(d_p2), G.ptr(d_ms), n, 0, 0, 1, 7, None)
+    import torch
+    G.sync()
+    assert torch.equal(d_p, d_p2)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+def test_global_norm_and_sum(precision):
+    L = G.lib(precision)
+    import torch
+    n, slices, stride = 100003, 4, 100003 + 5
+    x = G.rounded(rnd(stride * slices, 0, 1e-3), precision)       # dev/cuda/global_norm.cu scales inputs by 1e-3
+    d_x = G.dev(x, precision)
+    ns = (C.c_int * 2)(1, slices)
+    mx = L.llmk_get_max_num_block_sums(ns, 2)
+    out = torch.full((mx,), 5.0, dtype=torch.float32, device="cuda")
+    L.llmk_global_norm_squared(G.ptr(out), G.ptr(d_x), n, stride, slices, mx, 1, None)
+    L.llmk_global_norm_squared(G.ptr(out), G.ptr(d_x), 777, 0, 1, mx, 0, None)      # accumulates without reset
+    res = torch.zeros(1, dtype=torch.float32, device="cuda")
+    L.llmk_global_sum_deterministic(G.ptr(res), G.ptr(out), mx, None)
+    want = sum(ol.cref().cref_sum_squares(np.ascontiguousarray(x[s * stride:s * stride + n]), n) for s in range(slices))
+    want += ol.cref().cref_sum_squares(np.ascontiguousarray(x[:777]), 777)
+    assert abs(G.host(res)[0] - want) <= 1e-5 * want                               # dev/cuda/global_norm.cu: 1e-2
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+def test_shape_preconditions_are_reported(precision):
+    L = G.lib(precision)
+    L.llmk_set_error_mode(1)
+    try:
+        import torch
+        buf = torch.zeros(4096, dtype=G.torch_dtype(precision), device="cuda")
+        L.llmk_layernorm_forward(G.ptr(buf), None, None, G.ptr(buf), G.ptr(buf), G.ptr(buf), 1, 2, 67, None)
+        assert b"multiple" in L.llmk_last_error()
+        L.llmk_clear_error()
+        L.llmk_attention_forward(G.ptr(buf), None, G.ptr(buf), 1, 4, 3, 100, None)
+        assert L.llmk_last_error() != b""
+        L.llmk_clear_error()
+        L.llmk_gelu_forward(G.ptr(buf), G.ptr(buf), 0, None)                       # empty input: no-op, no error
+        assert L.llmk_last_error() == b""
+    finally:
+        L.llmk_clear_error()
+        L.llmk_set_error_mode(0)

@@ -1,0 +1,266 @@
+"""Whole training step through the host driver (include/llmk_gpt2.h) on the GPU against the CPU oracle,
+in the shape of the reference's test_gpt2.cu: logits / loss / every gradient tensor at step 0, ten
+AdamW-step losses, then checkpoint + state round trip with bit-identical resume (test_gpt2.cu:326-367).
+
+Tolerances are the ones the task states for this path:
+  fp32 library: loss within 1e-5 relative of the CPU loss, gradients within 1e-3 (per tensor, max|diff|/max|ref|)
+  bf16 library: |loss_gpu - loss_cpu| <= 2e-2 at each of 10 AdamW steps
+"""
+import ctypes as C
+import os
+
+import numpy as np
+import pytest
+
+import gpu_lib as G
+import oracle_lib as ol
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tiny_gpt2.npz")
+NAMES = ["wte", "wpe", "ln1w", "ln1b", "qkvw", "qkvb", "attprojw", "attprojb", "ln2w", "ln2b", "fcw", "fcb",
+         "fcprojw", "fcprojb", "lnfw", "lnfb"]
+
+
+class Model:
+    """Thin holder around the opaque driver handle."""
+
+    def __init__(self, precision, cfg, B, T, params=None, seed=42, master=1, recompute=1, gelu_fusion=0, checkpoint=None,
+                 weight_init=1):
+        self.L = G.lib(precision)
+        self.h = self.L.gpt2_create()
+        self.L.gpt2_set_options(self.h, master, recompute, gelu_fusion)
+        if checkpoint is not None:
+            self.L.gpt2_build_from_checkpoint(self.h, checkpoint.encode(), weight_init)
+        else:
+            self.L.gpt2_build_from_config(self.h, cfg.max_seq_len, cfg.vocab_size, cfg.padded_vocab_size, cfg.num_layers,
+                                          cfg.num_heads, cfg.channels, seed)
+        self.n = self.L.gpt2_num_parameters(self.h)
+        if params is not None:
+            self.L.gpt2_set_params_f32(self.h, params.ctypes.data_as(C.c_void_p))
+        self.L.gpt2_allocate_state(self.h, B, T)
+        self.B, self.T = B, T
+
+    def params(self):
+        out = np.zeros(self.n, np.float32)
+        self.L.gpt2_get_params_f32(self.h, out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def grads(self):
+        out = np.zeros(self.n, np.float32)
+        self.L.gpt2_get_grads_f32(self.h, out.ctypes.data_as(C.c_void_p))
+        return out
+
+    def logits(self, Vp):
+        out = np.zeros(self.B * self.T * Vp, np.float32)
+        self.L.gpt2_get_logits_f32(self.h, out.ctypes.data_as(C.c_void_p), self.B, self.T)
+        return out
+
+    def step(self, inp, tgt, t, lr, b1, b2, eps, wd, clip=0.0):
+        L, h = self.L, self.h
+        L.gpt2_forward(h, inp.ctypes.data_as(C.c_void_p), self.B, self.T)
+        L.gpt2_backward_and_reduce(h, inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p), 1, 0)
+        loss = L.gpt2_mean_loss(h)
+        norm = L.gpt2_calculate_grad_norm(h)
+        scale = 1.0 if (clip <= 0 or norm <= clip) else clip / norm
+        L.gpt2_update(h, lr, b1, b2, eps, wd, scale, t, 0)
+        return loss, norm
+
+    def free(self):
+        self.L.gpt2_free(self.h)
+        self.h = None
+
+
+def per_tensor_rel(a, b, sizes):
+    offs = np.cumsum([0] + sizes)
+    out = []
+    for i in range(16):
+        x, y = a[offs[i]:offs[i + 1]], b[offs[i]:offs[i + 1]]
+        out.append(float(np.abs(x - y).max() / max(np.abs(y).max(), 1e-30)))
+    return out
+
+
+def test_seeded_init_matches_oracle_init():
+    cfg = ol.Config(32, 100, 128, 2, 2, 128)
+    m = Model("fp32", cfg, 2, 32, seed=42)
+    np.testing.assert_allclose(m.params(), ol.init_params(cfg, 42), rtol=0, atol=1e-8)
+    m.free()
+    m = Model("bf16", cfg, 2, 32, seed=42)
+    np.testing.assert_array_equal(m.params(), G.rounded(ol.init_params(cfg, 42), "bf16"))
+    m.free()
+
+
+def test_fp32_tiny_model_against_reference_fixture():
+    g = np.load(GOLD)
+    cfg = ol.Config(*[int(x) for x in g["config"]])
+    B, T, steps = int(g["B"]), int(g["T"]), int(g["steps"])
+    lr, b1, b2, eps, wd = [float(x) for x in g["hyper"]]
+    params = ol.init_params(cfg, int(g["seed"]))
+    inp, tgt = np.ascontiguousarray(g["inputs"]), np.ascontiguousarray(g["targets"])
+    m = Model("fp32", cfg, B, T, params=params, master=0)
+    losses = []
+    for s in range(steps):
+        if s == 0:
+            m.L.gpt2_forward(m.h, inp.ctypes.data_as(C.c_void_p), B, T)
+            lg = m.logits(cfg.padded_vocab_size)
+            np.testing.assert_allclose(lg[g["logits_idx"]], g["logits_val"], rtol=1e-4, atol=1e-4)
+        loss, _ = m.step(inp, tgt, s + 1, lr, b1, b2, eps, wd)
+        if s == 0:
+            gr = m.grads()
+            scale = np.abs(g["grad_val_step0"]).max()
+            assert np.abs(gr[g["grad_idx"]] - g["grad_val_step0"]).max() <= 1e-3 * scale
+        losses.append(loss)
+    np.testing.assert_allclose(losses, g["losses"], rtol=1e-5)
+    m.free()
+
+
+@pytest.mark.parametrize("recompute,gelu_fusion", [(0, 0), (1, 2), (2, 1)])
+def test_fp32_small_model_vs_oracle_all_modes(recompute, gelu_fusion):
+    # 3 layers, 3 heads of 64, ragged T: every recompute / GELU-fusion combination gives the same numbers
+    cfg = ol.Config(64, 300, 320, 3, 3, 192)
+    B, T = 3, 40
+    params = ol.init_params(cfg, 5)
+    params += (np.random.RandomState(1).standard_normal(params.size) * 0.02).astype(np.float32)   # non-zero biases
+    sizes, _ = ol.param_sizes(cfg)
+    wte = params[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels); wte[cfg.vocab_size:] = 0
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 3)
+    ref = ol.cref_train(cfg, params, inp, tgt, B, T, 4, lr=1e-3, wd=0.1, wd_mask_2d=1, grad_clip=1.0, grad_step=0, want_logits=True)
+    m = Model("fp32", cfg, B, T, params=params, master=1, recompute=recompute, gelu_fusion=gelu_fusion)
+    for s in range(4):
+        loss, norm = m.step(inp, tgt, s + 1, 1e-3, 0.9, 0.999, 1e-8, 0.1, clip=1.0)
+        assert abs(loss - ref["losses"][s]) <= 1e-5 * abs(ref["losses"][s]), (s, loss, ref["losses"][s])
+        assert abs(norm - ref["gradnorm"][s]) <= 1e-4 * ref["gradnorm"][s]
+        if s == 0:
+            rel = per_tensor_rel(m.grads(), ref["grads"], sizes)
+            assert max(rel) <= 1e-3, dict(zip(NAMES, rel))
+    np.testing.assert_allclose(m.params(), ref["params"], rtol=1e-3, atol=3e-4)
+    m.free()
+
+
+def gpt2_124m():
+    return ol.Config(1024, 50257, 50304, 12, 12, 768)
+
+
+@pytest.fixture(scope="module")
+def config0_oracle():
+    """BASELINE config 0 on the CPU oracle: 124M, B=4, T=64, lr 1e-4, betas 0.9/0.999, wd 0, 10 steps."""
+    cfg = gpt2_124m()
+    params = ol.init_params(cfg, 42)
+    inp, tgt = ol.make_tokens(4, 64, cfg.vocab_size, 1337)
+    ref = ol.cref_train(cfg, params, inp, tgt, 4, 64, 10, lr=1e-4, b1=0.9, b2=0.999, eps=1e-8, wd=0.0, grad_step=0)
+    return cfg, params, inp, tgt, ref
+
+
+def test_fp32_gpt2_124m_config0(config0_oracle):
+    cfg, params, inp, tgt, ref = config0_oracle
+    sizes, _ = ol.param_sizes(cfg)
+    m = Model("fp32", cfg, 4, 64, params=params, master=0)
+    for s in range(10):
+        loss, _ = m.step(inp, tgt, s + 1, 1e-4, 0.9, 0.999, 1e-8, 0.0)
+        assert abs(loss - ref["losses"][s]) <= 1e-5 * abs(ref["losses"][s]), (s, loss, ref["losses"][s])
+        if s == 0:
+            rel = per_tensor_rel(m.grads(), ref["grads"], sizes)
+            assert max(rel) <= 1e-3, dict(zip(NAMES, rel))
+    # padded vocabulary rows stay exactly zero
+    wte = m.params()[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels)
+    assert (wte[cfg.vocab_size:] == 0).all()
+    m.free()
+
+
+def test_bf16_gpt2_124m_config0_tracks_cpu_loss(config0_oracle):
+    cfg, params, inp, tgt, ref = config0_oracle
+    sizes, _ = ol.param_sizes(cfg)
+    m = Model("bf16", cfg, 4, 64, params=params, master=1)
+    gpu_losses = []
+    for s in range(10):
+        loss, _ = m.step(inp, tgt, s + 1, 1e-4, 0.9, 0.999, 1e-8, 0.0)
+        gpu_losses.append(loss)
+        if s == 0:
+            # reference-style bf16 gradient check (test_gpt2.cu:274-278): |diff| <= tol + 0.079*|ref| on most elements
+            gr, rg = m.grads(), ref["grads"]
+            offs = np.cumsum([0] + sizes)
+            for i in range(16):
+                x, y = gr[offs[i]:offs[i + 1]], rg[offs[i]:offs[i + 1]]
+                assert np.abs(x - y).max() <= 0.05 * np.abs(y).max() + 1e-4, NAMES[i]
+    assert np.abs(np.array(gpu_losses) - ref["losses"]).max() <= 2e-2, (gpu_losses, ref["losses"])
+    wte = m.params()[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels)
+    assert (wte[cfg.vocab_size:] == 0).all()
+    m.free()
+
+
+@pytest.mark.parametrize("precision", ["bf16", "fp32"])
+def test_checkpoint_and_state_resume_is_bit_identical(precision, tmp_path):
+    cfg = ol.Config(64, 300, 320, 2, 2, 128)
+    B, T = 2, 64
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 11)
+    hp = (3e-3, 0.9, 0.95, 1e-8, 0.1)
+    m = Model(precision, cfg, B, T, seed=9, master=1)
+    for s in range(3):
+        m.step(inp, tgt, s + 1, *hp, clip=1.0)
+    ck, stt = str(tmp_path / "model.bin"), str(tmp_path / "state.bin")
+    m.L.gpt2_write_to_checkpoint(m.h, ck.encode())
+    m.L.gpt2_save_state(m.h, stt.encode(), 3)
+    first = [m.step(inp, tgt, s + 1, *hp, clip=1.0) for s in range(3, 6)]
+    p_first = m.params()
+    m.free()
+    # header of the model file follows the reference layout (train_gpt2.cu:435-446)
+    hdr = np.fromfile(ck, dtype=np.int32, count=256)
+    assert hdr[0] == 20240326 and hdr[1] == (5 if precision == "bf16" else 3)
+    assert list(hdr[2:8]) == [64, 300, 2, 2, 128, 320]
+    assert os.path.getsize(ck) == 1024 + sum(ol.param_sizes(cfg)[0]) * (2 if precision == "bf16" else 4)
+    shdr = np.fromfile(stt, dtype=np.int32, count=256)
+    assert shdr[0] == 20240527 and shdr[1] == 1 and shdr[4] == 1 and shdr[10] == 3
+    assert os.path.getsize(stt) == 1024 + 3 * 4 * sum(ol.param_sizes(cfg)[0])
+    # resume: weights are NOT read from the model file but re-derived from the fp32 master copy in the state file
+    m2 = Model(precision, cfg, B, T, master=1, checkpoint=ck, weight_init=0)
+    step = C.c_int(0)
+    m2.L.gpt2_load_state(m2.h, stt.encode(), C.byref(step))
+    assert step.value == 3
+    again = [m2.step(inp, tgt, s + 1, *hp, clip=1.0) for s in range(3, 6)]
+    assert again == first                                   # bit-identical losses and norms
+    np.testing.assert_array_equal(m2.params(), p_first)
+    m2.free()
+    if precision == "fp32":
+        # the fp32 model file is readable by the reference CPU trainer's loader rules: version 3
+        m3 = Model(precision, cfg, B, T, master=0, checkpoint=ck, weight_init=1)
+        assert m3.n == sum(ol.param_sizes(cfg)[0])
+        m3.free()
+
+
+def test_validate_matches_training_forward_loss():
+    cfg = ol.Config(64, 300, 320, 2, 2, 128)
+    B, T = 2, 64
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 5)
+    m = Model("bf16", cfg, B, T, seed=3)
+    val = m.L.gpt2_validate(m.h, inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p), B, T)
+    per_tok = np.ctypeslib.as_array(m.L.gpt2_cpu_losses(m.h), shape=(B * T,)).copy()
+    loss, _ = m.step(inp, tgt, 1, 0.0, 0.9, 0.95, 1e-8, 0.0)
+    assert abs(val - loss) < 1e-5
+    assert abs(per_tok.mean() - val) < 1e-5
+    # smaller batch / shorter sequence than allocated is allowed for inference (train_gpt2.cu:664-669)
+    v2 = m.L.gpt2_validate(m.h, inp[:32].ctypes.data_as(C.c_void_p), tgt[:32].ctypes.data_as(C.c_void_p), 1, 32)
+    assert abs(v2 - per_tok[:32].mean()) < 2e-2
+    mfu = m.L.gpt2_estimate_mfu(m.h, B * T, 1.0)
+    assert 0 < mfu < 1e-3
+    m.free()
+
+
+def test_bf16_full_size_step_properties():
+    """B=64, T=1024, 124M: the shape the throughput is quoted on. The oracle cannot run it, so check
+    what must hold at any size: initial loss ~ ln(V), loss decreases on a repeated batch, finite gradient norm,
+    padded wte rows untouched."""
+    cfg = gpt2_124m()
+    B, T = 64, 1024
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 99)
+    m = Model("bf16", cfg, B, T, seed=42)
+    losses = []
+    for s in range(3):
+        loss, norm = m.step(inp, tgt, s + 1, 6e-4, 0.9, 0.95, 1e-8, 0.1, clip=1.0)
+        assert np.isfinite(loss) and np.isfinite(norm) and norm > 0
+        losses.append(loss)
+    assert abs(losses[0] - np.log(cfg.vocab_size)) < 0.2
+    assert losses[2] < losses[0]
+    sizes, _ = ol.param_sizes(cfg)
+    wte = m.params()[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels)
+    assert (wte[cfg.vocab_size:] == 0).all()
+    m.free()
