@@ -5,7 +5,7 @@ fp32 library: tolerances of the reference's own kernel harness (dev/cuda/*.cu, 1
 bf16 library: the oracle is fed the bf16-rounded inputs; outputs may differ by bf16 rounding of the
 result (relative 2^-8) plus fp32 accumulation-order noise.
 """
-import ctypes as C
+import ctypes as CT
 
 import numpy as np
 import pytest
@@ -24,7 +24,7 @@ def rnd(shape, seed, scale=1.0):
 
 def tol(precision, fp32_atol, bf16_rel=1.0 / 128, bf16_atol=None):
     if precision == "fp32":
-        return dict(rtol=1e-5, atol=fp32_atol)
+        return dict(rtol=3e-5, atol=fp32_atol)
     return dict(rtol=bf16_rel, atol=bf16_atol if bf16_atol is not None else fp32_atol)
 
 
@@ -73,16 +73,16 @@ def test_encoder_backward(precision, B, T, C, V):
     scratch = torch.zeros(N * ncg * 20 + 64, dtype=torch.uint8, device="cuda")
     wl = np.zeros(N * ncg, np.int32); bk = np.zeros(4 * N * ncg, np.int32)
     d_wte, d_wpe, d_dout, d_inp = G.dev(dwte0, precision), G.dev(dwpe0, precision), G.dev(dout, precision), G.dev(inp)
-    L.llmk_encoder_backward(G.ptr(d_wte), G.ptr(d_wpe), G.ptr(scratch), wl.ctypes.data_as(C.c_void_p),
-                            bk.ctypes.data_as(C.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(C.c_void_p),
+    L.llmk_encoder_backward(G.ptr(d_wte), G.ptr(d_wpe), G.ptr(scratch), wl.ctypes.data_as(CT.c_void_p),
+                            bk.ctypes.data_as(CT.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(CT.c_void_p),
                             B, T, C, 1234, None)
     # stochastic rounding lands on one of the two bf16 neighbours of the exact sum: 1 ulp = 2^-7 relative
     close(G.host(d_wte), rwte, **tol(precision, 1e-4, bf16_rel=1.0 / 64, bf16_atol=2e-2), what="dwte")
     close(G.host(d_wpe), rwpe, **tol(precision, 1e-4, bf16_rel=1.0 / 64, bf16_atol=2e-2), what="dwpe")
     # determinism: same call, same bits
     d_wte2, d_wpe2 = G.dev(dwte0, precision), G.dev(dwpe0, precision)
-    L.llmk_encoder_backward(G.ptr(d_wte2), G.ptr(d_wpe2), G.ptr(scratch), wl.ctypes.data_as(C.c_void_p),
-                            bk.ctypes.data_as(C.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(C.c_void_p),
+    L.llmk_encoder_backward(G.ptr(d_wte2), G.ptr(d_wpe2), G.ptr(scratch), wl.ctypes.data_as(CT.c_void_p),
+                            bk.ctypes.data_as(CT.c_void_p), G.ptr(d_dout), G.ptr(d_inp), inp.ctypes.data_as(CT.c_void_p),
                             B, T, C, 1234, None)
     G.sync()
     assert torch.equal(d_wte, d_wte2) and torch.equal(d_wpe, d_wpe2)
@@ -197,7 +197,15 @@ def test_fused_classifier(precision, N, V, P):
     L.llmk_fused_classifier(G.ptr(d_z), G.ptr(d_l), dloss, G.ptr(d_t), 1, N, V, P, 1, None)
     close(G.host(d_l), rl, rtol=1e-5, atol=1e-4)                                  # classifier_fused.cu:739
     out = G.host(d_z)
-    close(out[:, :V], rd[:, :V], **tol(precision, 1e-6, bf16_rel=1.0 / 64, bf16_atol=1e-5), what="dlogits")
+    # the oracle adds its 50k exponentials one after the other in fp32 (train_gpt2.c:468-472), which costs it up to
+    # ~1e-4 relative; a float64 softmax shows which side is exact: oracle within 1e-3 of it, GPU within 2e-5
+    z64 = z[:, :V].astype(np.float64)
+    p64 = np.exp(z64 - z64.max(1, keepdims=True)); p64 /= p64.sum(1, keepdims=True)
+    p64[np.arange(N), tg] -= 1.0
+    close(rd[:, :V], p64 * dloss, rtol=1e-3, atol=1e-7, what="oracle vs float64")
+    close(out[:, :V], p64 * dloss, **tol(precision, 1e-7, bf16_rel=1.0 / 64, bf16_atol=1e-5), what="dlogits")
+    if precision == "fp32":
+        close(out[:, :V], p64 * dloss, rtol=3e-5, atol=1e-7, what="dlogits vs float64")
     np.testing.assert_array_equal(out[:, V:], z[:, V:])
     G.check_no_error(L)
 
@@ -428,7 +436,7 @@ def test_global_norm_and_sum(precision):
     n, slices, stride = 100003, 4, 100003 + 5
     x = G.rounded(rnd(stride * slices, 0, 1e-3), precision)       # dev/cuda/global_norm.cu scales inputs by 1e-3
     d_x = G.dev(x, precision)
-    ns = (C.c_int * 2)(1, slices)
+    ns = (CT.c_int * 2)(1, slices)
     mx = L.llmk_get_max_num_block_sums(ns, 2)
     out = torch.full((mx,), 5.0, dtype=torch.float32, device="cuda")
     L.llmk_global_norm_squared(G.ptr(out), G.ptr(d_x), n, stride, slices, mx, 1, None)
