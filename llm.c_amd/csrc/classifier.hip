@@ -65,8 +65,12 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
         if (v < nvalid) {
             bool has_target = (target / VN) == v;
             if (has_target) {
-                // -log softmax[target] = (max - logit) + log(sum); accumulates like the reference (:81)
-                float lt = to_f32(r[i][target % VN]);
+                // -log softmax[target] = (max - logit) + log(sum); accumulates like the reference (:81).
+                // Compare-select instead of r[i][target % VN]: a run-time index would push the row out of registers.
+                float lt = 0.f;
+#pragma unroll
+                for (int k = 0; k < VN; k++)
+                    if (k == target % VN) lt = to_f32(r[i][k]);
                 losses[row] += (mx - lt) + logf(sum);
             }
             if (WRITE) {
