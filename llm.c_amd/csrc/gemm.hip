@@ -26,29 +26,11 @@
 // used for 1e-5 parity against the CPU reference.
 #include "common.hpp"
 #include "gelu.hpp"
+#include "gemm_pipelined.hpp"
 #include "../../include/llmk.h"
 
 namespace {
-
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
-typedef __attribute__((ext_vector_type(4))) short s16x4;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
-
-enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5 };
-
-struct GemmArgs {
-    const floatX* A;
-    const floatX* B;
-    floatX* C;
-    int M, N, K;          // C[M][N] = sum_k A(m,k) * B(n,k)
-    int lda, ldb, ldc;    // leading dimensions of the stored matrices, in elements
-    const floatX* bias;   // [N] or nullptr                         (EPI_BIAS*)
-    floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU)
-    float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL)
-    int k_per_split;      // multiple of the K step
-};
+using namespace gemmk;
 
 constexpr int GROUP_M = 8;
 
@@ -277,6 +259,38 @@ void launch_gemm(const GemmArgs& g, int splits, bool big, hipStream_t st) {
 constexpr int K_ALIGN = 8;       // K-contiguous rows are read in 16-byte chunks
 constexpr int BIG_TILE = 256, SMALL_TILE = 128, K_STEP = 64;
 
+// Persistent direct-to-LDS kernel (gemm_pipelined.hpp). Preconditions: K and the per-split K multiples of 32,
+// leading dimensions and N multiples of 8, 16-byte aligned operands, 8-byte aligned bias.
+bool pipelined_ok(const GemmArgs& g) {
+    auto al = [](const void* p, uintptr_t a) { return ((uintptr_t)p % a) == 0; };
+    return g.K % PBK == 0 && g.k_per_split % PBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 8 == 0 &&
+           g.N % 8 == 0 && al(g.A, 16) && al(g.B, 16) && al(g.C, 16) && (!g.bias || al(g.bias, 8)) && (!g.aux || al(g.aux, 16));
+}
+template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
+void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
+    constexpr int NW = WGM * WGN;
+    constexpr int STAGE = (BM + BN) * PBK * 2;
+    constexpr int STRIP = 32 * EPI_PITCH;
+    constexpr int IN_SLOT = STAGE / STRIP;
+    constexpr int SMEM = STAGES * STAGE + (NW > IN_SLOT ? (NW - IN_SLOT) * STRIP : 0);
+    auto kern = gemm_pipelined_kernel<BM, BN, WGM, WGN, A_T, B_T, EPI>;
+    static bool attr_set = false;
+    if (!attr_set) {
+        HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM));
+        attr_set = true;
+    }
+    g.splits = splits;
+    const int work = CEIL_DIV(g.M, BM) * CEIL_DIV(g.N, BN) * splits;
+    const int grid = min(work, llmk::device_info().num_cu);
+    kern<<<grid, NW * 64, SMEM, st>>>(g);
+    LAUNCH_CHECK();
+}
+template <bool A_T, bool B_T, int EPI>
+void launch_pipelined(const GemmArgs& g, int splits, bool big, hipStream_t st) {
+    if (big) launch_pipelined_cfg<256, 256, 2, 4, A_T, B_T, EPI>(g, splits, st);
+    else launch_pipelined_cfg<128, 128, 2, 2, A_T, B_T, EPI>(g, splits, st);
+}
+
 #else
 // =============================================================================================
 // fp32 MFMA kernel (parity mode): 128x128 tile, K step 16, 4 waves of 64x64
@@ -497,6 +511,9 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
         llmk_gelu_forward(out, pre_gelu, M * OC, stream);
     } else {
         g.C = (floatX*)out;
+#if !defined(LLMK_FP32)
+        if (pipelined_ok(g)) { launch_pipelined<false, false, EPI_BIAS>(g, 1, big, st); return; }
+#endif
         launch_gemm<false, false, EPI_BIAS>(g, 1, big, st);
     }
 }
@@ -538,6 +555,10 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                                  ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
             if (fused) {
                 g.aux = (floatX*)pre_gelu;
+#if !defined(LLMK_FP32)
+                if (pipelined_ok(g)) launch_pipelined<false, true, EPI_DGELU>(g, 1, big, st);
+                else
+#endif
                 launch_gemm<false, true, EPI_DGELU>(g, 1, big, st);
             } else {
                 launch_gemm<false, true, EPI_STORE>(g, 1, big, st);
