@@ -23,8 +23,10 @@ KERNEL_SOURCES = ["runtime.hip", "layernorm.hip", "gelu.hip", "encoder.hip", "cl
 DRIVER_SOURCES = ["gpt2.cpp"]
 
 # -packed-fp32-ops off: this toolchain's packed fp32 instructions are not trusted on this hardware pool
+# -amdgpu-mfma-vgpr-form: keep MFMA accumulators in ordinary VGPRs. The softmax between the two MFMA groups of the
+# attention kernels works on accumulator values; with AGPR accumulators every value is copied out and back.
 COMMON = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
-          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 PREC_DEFS = {"bf16": [], "fp32": ["-DLLMK_FP32"]}
 
 

@@ -153,36 +153,41 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
                         sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32 * kb, s, lane), qf[s], sacc[kb], 0, 0, 0);
                 }
             }
-            const bool diag = 64 * j + 63 > qw0;          // some (key, query) pairs of this tile are masked
+            if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int key = 64 * j + 32 * kb + acc_row(r, lane);
+                        if (key > my_q) sacc[kb][r] = -INFINITY;
+                    }
+            }
             float mx = -INFINITY;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    if (diag) {
-                        const int key = 64 * j + 32 * kb + acc_row(r, lane);
-                        if (key > my_q) sacc[kb][r] = -INFINITY;
-                    }
-                    mx = fmaxf(mx, sacc[kb][r]);
-                }
+                for (int r = 0; r < 16; r++) mx = fmaxf(mx, sacc[kb][r]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float m_new = fmaxf(m, mx * c);
-            const float alpha = fast_exp2(m - m_new);
-            m = m_new;
+            if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // some row's running max moved: rescale (rare after the first tiles)
+                const float alpha = fast_exp2(m - m_new);
+                m = m_new;
+                l *= alpha;
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+            }
             float rs = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) {
-                    float p = fast_exp2(fmaf(sacc[kb][r], c, -m_new));
+                    float p = fast_exp2(fmaf(sacc[kb][r], c, -m));
                     sacc[kb][r] = p;
                     rs += p;
                 }
-            l = l * alpha + rs;
-#pragma unroll
-            for (int d = 0; d < 2; d++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+            l += rs;
 #pragma unroll
             for (int s2 = 0; s2 < 4; s2++) {
                 if (s2 < 2 || kb1) {
@@ -320,22 +325,26 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s, lane), vf[s], pacc, 0, 0, 0);
             }
-            const bool diag = q0 < kw0 + 31;
+            f32x4 d4[4];
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int rr = 32 * qb + g * 8 + half * 4;
                 const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[buf][rr]);
-                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
+                d4[g] = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int r = 4 * g + e;
-                    float p = fast_exp2(fmaf(sacc[r], c, -l4[e]));
-                    const int q = 64 * qi + rr + e;
-                    if ((diag && q < my_k) || q >= T) p = 0.f;
-                    sacc[r] = p;
-                    pacc[r] = p * (pacc[r] - d4[e]);
+                for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+            }
+            if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int q = q0 + acc_row(r, lane);
+                    if (q < my_k || q >= T) sacc[r] = 0.f;
                 }
             }
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[g][e]);
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
                 const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
@@ -432,13 +441,15 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32 * kb, s, lane), qf[s], sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tv, 32 * kb, s, lane), dof[s], pacc, 0, 0, 0);
             }
-            const bool diag = k0 + 31 > qw0;
 #pragma unroll
-            for (int r = 0; r < 16; r++) {
-                float p = fast_exp2(fmaf(sacc[r], c, -lse2));
-                if (diag && (k0 + acc_row(r, lane) > my_q)) p = 0.f;
-                pacc[r] = p * (pacc[r] - dsum);
+            for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
+            if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (k0 + acc_row(r, lane) > my_q) sacc[r] = 0.f;
             }
+#pragma unroll
+            for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
                 const bf16x8 dsf = pack_acc(pacc, s2);
