@@ -270,9 +270,7 @@ template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
 void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
     constexpr int NW = WGM * WGN;
     constexpr int STAGE = (BM + BN) * PBK * 2;
-    constexpr int STRIP = 32 * EPI_PITCH;
-    constexpr int IN_SLOT = STAGE / STRIP;
-    constexpr int SMEM = STAGES * STAGE + (NW > IN_SLOT ? (NW - IN_SLOT) * STRIP : 0);
+    constexpr int SMEM = STAGES * STAGE;
     auto kern = gemm_pipelined_kernel<BM, BN, WGM, WGN, A_T, B_T, EPI>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -289,6 +287,12 @@ template <bool A_T, bool B_T, int EPI>
 void launch_pipelined(const GemmArgs& g, int splits, bool big, hipStream_t st) {
     if (big) launch_pipelined_cfg<256, 256, 2, 4, A_T, B_T, EPI>(g, splits, st);
     else launch_pipelined_cfg<128, 128, 2, 2, A_T, B_T, EPI>(g, splits, st);
+}
+// pipelined kernel when its preconditions hold, generic kernel otherwise
+template <bool A_T, bool B_T, int EPI>
+void launch_best(const GemmArgs& g, int splits, bool big, hipStream_t st) {
+    if (pipelined_ok(g)) launch_pipelined<A_T, B_T, EPI>(g, splits, big, st);
+    else launch_gemm<A_T, B_T, EPI>(g, splits, big, st);
 }
 
 #else
@@ -414,6 +418,8 @@ void launch_gemm(const GemmArgs& g, int splits, bool /*big*/, hipStream_t st) {
 }
 constexpr int K_ALIGN = 4;
 constexpr int BIG_TILE = 128, SMALL_TILE = 128, K_STEP = 16;
+template <bool A_T, bool B_T, int EPI>
+void launch_best(const GemmArgs& g, int splits, bool big, hipStream_t st) { launch_gemm<A_T, B_T, EPI>(g, splits, big, st); }
 #endif
 
 // C[m][n] (+)= sum over splits of partial[s][m][n], in split order
@@ -436,9 +442,11 @@ splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, 
 }
 
 // ---- bias gradient: column sums of dout[N][OC] -----------------------------------------------
-// workgroup = 32 column-vectors x 8 row lanes; grid.y splits the rows so the machine is full.
+// HBM-bound streaming reduction. Workgroup = 32 column-vectors (512 B of a row) x 8 row lanes; each lane keeps
+// four row loads in flight. grid.y splits the rows so that ~2 workgroups per CU are resident; their partial sums
+// go to the caller's fp32 scratch and are added in a fixed order by a second, tiny kernel (no atomics).
 constexpr int VN = vecX::N;
-constexpr int BG_COLV = 32, BG_ROWL = 8;
+constexpr int BG_COLV = 32, BG_ROWL = 8, BG_UNROLL = 4;
 __global__ void __launch_bounds__(256)
 bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, int N, int OC) {
     __shared__ float red[BG_ROWL][BG_COLV * VN + 1];
@@ -448,8 +456,19 @@ bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, i
 #pragma unroll
     for (int k = 0; k < VN; k++) acc[k] = 0.f;
     if (col < OC) {
-        for (int r = blockIdx.y * BG_ROWL + rl; r < N; r += gridDim.y * BG_ROWL) {
-            vecX d = ld_vec(dout + (size_t)r * OC + col);
+        const int rstep = gridDim.y * BG_ROWL;
+        int r = blockIdx.y * BG_ROWL + rl;
+        for (; r + (BG_UNROLL - 1) * rstep < N; r += BG_UNROLL * rstep) {
+            vecX d[BG_UNROLL];
+#pragma unroll
+            for (int u = 0; u < BG_UNROLL; u++) d[u] = ld_vec_nt(dout + (size_t)(r + u * rstep) * OC + col);
+#pragma unroll
+            for (int u = 0; u < BG_UNROLL; u++)
+#pragma unroll
+                for (int k = 0; k < VN; k++) acc[k] += to_f32(d[u][k]);
+        }
+        for (; r < N; r += rstep) {
+            vecX d = ld_vec_nt(dout + (size_t)r * OC + col);
 #pragma unroll
             for (int k = 0; k < VN; k++) acc[k] += to_f32(d[k]);
         }
@@ -467,17 +486,29 @@ bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, i
         }
     }
 }
-__global__ void __launch_bounds__(256)
+// dbias[oc] += sum_y partial[y][oc]: 32 columns per workgroup, 8 groups each adding every 8th partial, then the
+// 8 sub-sums in group order
+constexpr int BGR_COLS = 32, BGR_GROUPS = 8;
+__global__ void __launch_bounds__(BGR_COLS * BGR_GROUPS)
 bias_grad_reduce_kernel(floatX* __restrict__ dbias, const float* __restrict__ partial, int OC, int ny) {
-    int oc = blockIdx.x * blockDim.x + threadIdx.x;
-    if (oc >= OC) return;
+    __shared__ float sub[BGR_GROUPS][BGR_COLS];
+    const int cl = threadIdx.x % BGR_COLS, grp = threadIdx.x / BGR_COLS;
+    const int oc = blockIdx.x * BGR_COLS + cl;
     float s = 0.f;
-    for (int y = 0; y < ny; y++) s += partial[(size_t)y * OC + oc];
-    dbias[oc] = from_f32<floatX>(to_f32(dbias[oc]) + s);
+    if (oc < OC)
+        for (int y = grp; y < ny; y += BGR_GROUPS) s += partial[(size_t)y * OC + oc];
+    sub[grp][cl] = s;
+    __syncthreads();
+    if (grp == 0 && oc < OC) {
+        float t = 0.f;
+#pragma unroll
+        for (int g2 = 0; g2 < BGR_GROUPS; g2++) t += sub[g2][cl];
+        dbias[oc] = from_f32<floatX>(to_f32(dbias[oc]) + t);
+    }
 }
 int bias_grad_ny(int OC) {
     int gx = CEIL_DIV(OC, BG_COLV * VN);
-    return max(1, llmk::device_info().num_cu * 4 / gx);
+    return max(1, llmk::device_info().num_cu * 2 / gx);
 }
 
 bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
@@ -503,18 +534,15 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
                          ((double)M * C + (double)OC * C + (double)M * OC) * sizeof(floatX), st);
     if (pre_gelu && gelu_fusion >= 1) {
         g.C = (floatX*)out; g.aux = (floatX*)pre_gelu;
-        launch_gemm<false, false, EPI_BIAS_GELU>(g, 1, big, st);
+        launch_best<false, false, EPI_BIAS_GELU>(g, 1, big, st);
     } else if (pre_gelu) {
         g.C = (floatX*)pre_gelu;
-        launch_gemm<false, false, EPI_BIAS>(g, 1, big, st);
+        launch_best<false, false, EPI_BIAS>(g, 1, big, st);
         if (prof.on) { llmk::prof_end(st); prof.on = false; }
         llmk_gelu_forward(out, pre_gelu, M * OC, stream);
     } else {
         g.C = (floatX*)out;
-#if !defined(LLMK_FP32)
-        if (pipelined_ok(g)) { launch_pipelined<false, false, EPI_BIAS>(g, 1, big, st); return; }
-#endif
-        launch_gemm<false, false, EPI_BIAS>(g, 1, big, st);
+        launch_best<false, false, EPI_BIAS>(g, 1, big, st);
     }
 }
 
@@ -538,7 +566,7 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         llmk::ProfScope prof("bias_grad", 0, (double)M * OC * sizeof(floatX), st);
         bias_grad_kernel<<<dim3(CEIL_DIV(OC, BG_COLV * VN), ny), 256, 0, st>>>(dbias_buffer, (const floatX*)dout, M, OC);
         LAUNCH_CHECK();
-        bias_grad_reduce_kernel<<<CEIL_DIV(OC, 256), 256, 0, st>>>((floatX*)dbias, dbias_buffer, OC, ny);
+        bias_grad_reduce_kernel<<<CEIL_DIV(OC, BGR_COLS), BGR_COLS * BGR_GROUPS, 0, st>>>((floatX*)dbias, dbias_buffer, OC, ny);
         LAUNCH_CHECK();
     }
 
@@ -555,13 +583,9 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                                  ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
             if (fused) {
                 g.aux = (floatX*)pre_gelu;
-#if !defined(LLMK_FP32)
-                if (pipelined_ok(g)) launch_pipelined<false, true, EPI_DGELU>(g, 1, big, st);
-                else
-#endif
-                launch_gemm<false, true, EPI_DGELU>(g, 1, big, st);
+                launch_best<false, true, EPI_DGELU>(g, 1, big, st);
             } else {
-                launch_gemm<false, true, EPI_STORE>(g, 1, big, st);
+                launch_best<false, true, EPI_STORE>(g, 1, big, st);
             }
         }
         if (pre_gelu && !fused) llmk_gelu_backward_inplace(dinp, pre_gelu, M * C, stream);
@@ -585,13 +609,13 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         const double tn_bytes = ((double)M * OC + (double)M * C + 2.0 * OC * C) * sizeof(floatX);
         if (splits == 1) {
             llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
-            launch_gemm<true, true, EPI_ACCUM>(g, 1, big, st);
+            launch_best<true, true, EPI_ACCUM>(g, 1, big, st);
         } else {
             const size_t mn = (size_t)OC * C;
             g.partial = (float*)llmk::workspace(mn * splits * sizeof(float));
             {
                 llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
-                launch_gemm<true, true, EPI_PARTIAL>(g, splits, big, st);
+                launch_best<true, true, EPI_PARTIAL>(g, splits, big, st);
             }
             llmk::ProfScope prof("splitk_reduce", 0, (double)mn * splits * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
             splitk_reduce_kernel<true><<<(unsigned)CEIL_DIV(mn / 4, (size_t)256), 256, 0, st>>>((floatX*)dweight, g.partial, mn, splits);

@@ -9,17 +9,17 @@
 //     classic "global -> registers -> ds_write" staging leaves the matrix cores idle while every
 //     wave writes LDS. Here operands go global -> LDS directly (global_load_lds_dwordx4): no
 //     staging registers, no ds_write instructions, and the LDS writes trickle in while MFMAs run.
-//   * K advances in blocks of 32 through a ring of four 32 KiB LDS slots; loads run three blocks
-//     (96 KiB per CU) ahead of the math, which is what it takes to cover HBM/L2 latency at this
-//     consumption rate. One s_barrier per block.
+//   * K advances in blocks of 32 through a ring of five 32 KiB LDS slots (all 160 KiB of the CU); loads run
+//     four blocks (128 KiB per CU) ahead of the math, which is what it takes to cover HBM/L2 latency at
+//     this consumption rate. One s_barrier per block, without a memory fence (a fence would drain the ring).
 //   * A direct-to-LDS load deposits each wave's 64 x 16 B linearly, so the anti-bank-conflict
 //     swizzle is applied on the global side: lane p of a row fetches chunk p ^ f(row), and the
 //     MFMA operand reads undo it. K-contiguous tiles: [row][32] with f = (row>>2)&3 (ds_read_b128
 //     conflict-free). K-major tiles: [k][row] as in memory, f = 4*(k&3), read with the transposing
 //     ds_read_b64_tr_b16 so no software transpose is needed for dinp/dweight.
 //   * The kernel is persistent (one workgroup per CU walks a list of tiles). When a tile's K loop
-//     ends, the first three K-blocks of the NEXT tile are already requested into three ring slots
-//     while the epilogue runs out of the fourth slot plus the 32 KiB of LDS above the ring.
+//     ends, the first four K-blocks of the NEXT tile are requested into four ring slots while the
+//     epilogue stages its output through the fifth.
 //   * The MFMA is issued with swapped operands (D^T = B.A^T): each lane then owns 4 consecutive
 //     output columns of one row, which it writes as 8 bytes into a per-wave LDS staging strip; the
 //     strip is read back row-contiguously so that global stores (and the loads of pre_gelu / the
@@ -57,7 +57,7 @@ struct GemmArgs {
 #if !defined(LLMK_FP32)
 
 constexpr int PBK = 32;                 // K per pipeline block
-constexpr int STAGES = 4;
+constexpr int STAGES = 5;                // ring slots; loads run STAGES-1 K blocks ahead of the math
 constexpr int LDS_TOTAL = 160 * 1024;
 constexpr int EPI_PITCH = 144;          // bytes per staged output row: 128 + 16
 
@@ -99,7 +99,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int A_CHUNKS = A_STAGE / 1024, B_CHUNKS = B_STAGE / 1024;
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
-    static_assert(STAGES * STAGE + 32 * 1024 <= LDS_TOTAL || STAGE <= 16 * 1024, "LDS budget");
+    static_assert(STAGES * STAGE <= LDS_TOTAL, "LDS budget");
     static_assert(TN % 2 == 0, "epilogue strips are 64 columns wide");
     static_assert(A_CHUNKS % NW == 0, "each load slot of a wave must be all-A or all-B");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
@@ -172,15 +172,20 @@ gemm_pipelined_kernel(GemmArgs g) {
         const int row = row0 + idx, c = 2 * s + half;
         return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((c ^ ((row >> 2) & 3)) << 4));
     };
+    // The transposing reads are issued as inline asm on purpose: for the builtin, the compiler cannot tell that the
+    // read does not alias the in-flight direct-to-LDS loads and would wait for ALL of them (vmcnt(0)) first, which
+    // serialises loading and math. The price is that their completion has to be awaited by hand (lds_wait below).
     auto frag_t = [&](const char* tile, int pitch, int row0, int s) -> bf16x8 {   // K-major tile [k][row], transposing read
         const int s16 = lane & 15, grp = lane >> 4;
         const int krow = 16 * s + 8 * (grp >> 1) + (s16 >> 2);             // (krow & 3) is the same for krow + 4
         const int col = row0 + (grp & 1) * 16 + 4 * (s16 & 3);
         const int cn = (col >> 3) ^ (4 * (krow & 3));
         const char* p = tile + krow * pitch + cn * 16 + (col & 7) * 2;
-        typedef s16x4 __attribute__((address_space(3))) * lp;
-        s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(p));
-        s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(p + 4 * pitch));
+        const unsigned a0 = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
+        const unsigned a1 = a0 + 4 * pitch;
+        s16x4 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a0));
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi) : "v"(a1));
         union { struct { s16x4 a, b; } s; bf16x8 v; } u;
         u.s.a = lo; u.s.b = hi;
         return u.v;
@@ -213,7 +218,8 @@ gemm_pipelined_kernel(GemmArgs g) {
         // ---- K loop -----------------------------------------------------------------------------
         for (int kb = 0; kb < nkb; kb++) {
             const int ahead = min(STAGES - 2, nkb - 1 - kb);      // younger blocks that may stay in flight
-            if (ahead >= 2) wait_vmcnt<2 * CPW>();
+            if (ahead >= 3) wait_vmcnt<3 * CPW>();
+            else if (ahead == 2) wait_vmcnt<2 * CPW>();
             else if (ahead == 1) wait_vmcnt<CPW>();
             else wait_vmcnt<0>();
             barrier_no_fence();                                   // block kb landed for everyone; slot of kb-1 is free
@@ -227,6 +233,16 @@ gemm_pipelined_kernel(GemmArgs g) {
                 for (int i = 0; i < TM; i++) fa[i] = A_T ? frag_t(sa, BM * 2, wm * WTM + i * 32, s) : frag_k(sa, wm * WTM + i * 32, s);
 #pragma unroll
                 for (int j = 0; j < TN; j++) fb[j] = B_T ? frag_t(sb, BN * 2, wn * WTN + j * 32, s) : frag_k(sb, wn * WTN + j * 32, s);
+                if (A_T || B_T) {      // hand-issued reads: wait for LDS, with the operands tied to the wait so nothing moves above it
+                    if (A_T) {
+#pragma unroll
+                        for (int i = 0; i < TM; i++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[i]));
+                    }
+                    if (B_T) {
+#pragma unroll
+                        for (int j = 0; j < TN; j++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[j]));
+                    }
+                }
 #pragma unroll
                 for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -256,13 +272,12 @@ gemm_pipelined_kernel(GemmArgs g) {
         }
 
         // ---- epilogue ---------------------------------------------------------------------------------
-        // wave-private staging strip: 32 rows x (64 cols as 128 B + 16 B pad); the free ring slot holds
-        // STAGE / 4608 strips, the rest live in the 32 KiB above the ring
+        // wave-private staging strip inside the free ring slot: 16 rows x (128 B + 16 B pad)
         {
-            constexpr int STRIP = 32 * EPI_PITCH;
-            constexpr int IN_SLOT = STAGE / STRIP;
-            char* strip = wave < IN_SLOT ? lds + ring_free * STAGE + wave * STRIP
-                                         : lds + STAGES * STAGE + (wave - IN_SLOT) * STRIP;
+            constexpr int STRIP_ROWS = 16;
+            constexpr int STRIP = STRIP_ROWS * EPI_PITCH;
+            static_assert(NW * STRIP <= STAGE, "all strips must fit in one ring slot");
+            char* strip = lds + ring_free * STAGE + wave * STRIP;
             const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
             constexpr bool F32OUT = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
             constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
@@ -271,84 +286,90 @@ gemm_pipelined_kernel(GemmArgs g) {
             for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++) {
-                    // phase 1: lane (m = idx, half) owns n = 8q + 4*half + 0..3 of each 32-column block
 #pragma unroll
-                    for (int j = pass * JP; j < (pass + 1) * JP; j++) {
+                    for (int hsel = 0; hsel < 2; hsel++) {        // rows 0..15 / 16..31 of the 32-row block
+                        // phase 1: lane (m = idx, half) owns n = 8q + 4*half + 0..3 of each 32-column block
+                        if ((idx >> 4) == hsel) {
 #pragma unroll
-                        for (int q = 0; q < 4; q++) {
-                            const int nl = j * 32 + 8 * q + 4 * half;      // column inside the wave tile
-                            const int sl = (j - pass * JP) * 32 + 8 * q + 4 * half;   // column inside the strip
-                            float v[4];
+                            for (int j = pass * JP; j < (pass + 1) * JP; j++) {
 #pragma unroll
-                            for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
-                            if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
-                                if (g.bias) {
-                                    const int n = wn0 + nl;
-                                    if (n < g.N) {
-                                        bf16x4 b4 = *reinterpret_cast<const bf16x4*>(g.bias + n);
+                                for (int q = 0; q < 4; q++) {
+                                    const int nl = j * 32 + 8 * q + 4 * half;                 // column inside the wave tile
+                                    const int sl = (j - pass * JP) * 32 + 8 * q + 4 * half;   // column inside the strip
+                                    float v[4];
 #pragma unroll
-                                        for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
+                                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
+                                    if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+                                        if (g.bias) {
+                                            const int n = wn0 + nl;
+                                            if (n < g.N) {
+                                                bf16x4 b4 = *reinterpret_cast<const bf16x4*>(g.bias + n);
+#pragma unroll
+                                                for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
+                                            }
+                                        }
+                                    }
+                                    char* dst = strip + (idx & 15) * EPI_PITCH;
+                                    if (F32OUT) {
+                                        f32x4 o = {v[0], v[1], v[2], v[3]};
+                                        *reinterpret_cast<f32x4*>(dst + (8 * q + 4 * half) * 4) = o;
+                                    } else {
+                                        bf16x4 o;
+#pragma unroll
+                                        for (int e = 0; e < 4; e++) o[e] = (__bf16)v[e];
+                                        *reinterpret_cast<bf16x4*>(dst + sl * 2) = o;
                                     }
                                 }
                             }
+                        }
+                        __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): the strip is written
+                        __builtin_amdgcn_wave_barrier();
+                        // phase 2: 16 rows x 128 B, 8 lanes per row
+#pragma unroll
+                        for (int t = 0; t < 2; t++) {
+                            const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                            const int m = wm0 + i * 32 + hsel * 16 + row;
+                            u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * EPI_PITCH + ch * 16);
                             if (F32OUT) {
-                                f32x4 o = {v[0], v[1], v[2], v[3]};
-                                *reinterpret_cast<f32x4*>(strip + idx * EPI_PITCH + (8 * q + 4 * half) * 4) = o;
+                                const int n = wn0 + pass * 32 + ch * 4;
+                                if (m < g.M && n < g.N) {
+                                    if (EPI == EPI_PARTIAL) {
+                                        *reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n) = raw;
+                                    } else {
+                                        union { u32x4 u; f32x4 f; } x;
+                                        x.u = raw;
+                                        floatX* cp = g.C + (size_t)m * g.ldc + n;
+                                        bf16x4 old = *reinterpret_cast<const bf16x4*>(cp), o4;
+#pragma unroll
+                                        for (int e = 0; e < 4; e++) o4[e] = (__bf16)((float)old[e] + x.f[e]);
+                                        *reinterpret_cast<bf16x4*>(cp) = o4;
+                                    }
+                                }
                             } else {
-                                bf16x4 o;
-#pragma unroll
-                                for (int e = 0; e < 4; e++) o[e] = (__bf16)v[e];
-                                *reinterpret_cast<bf16x4*>(strip + idx * EPI_PITCH + sl * 2) = o;
-                            }
-                        }
-                    }
-                    __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): the strip is written
-                    __builtin_amdgcn_wave_barrier();
-                    // phase 2: 32 rows x 128 B, 8 lanes per row
-#pragma unroll
-                    for (int t = 0; t < 4; t++) {
-                        const int row = t * 8 + (lane >> 3), ch = lane & 7;
-                        const int m = wm0 + i * 32 + row;
-                        u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * EPI_PITCH + ch * 16);
-                        if (F32OUT) {
-                            const int n = wn0 + pass * 32 + ch * 4;
-                            if (m < g.M && n < g.N) {
-                                if (EPI == EPI_PARTIAL) {
-                                    *reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n) = raw;
-                                } else {
-                                    union { u32x4 u; f32x4 f; } x;
+                                const int n = wn0 + pass * 64 + ch * 8;
+                                if (m < g.M && n < g.N) {
+                                    const size_t o = (size_t)m * g.ldc + n;
+                                    union { u32x4 u; bf16x8 h; } x, y, z;
                                     x.u = raw;
-                                    floatX* cp = g.C + (size_t)m * g.ldc + n;
-                                    bf16x4 old = *reinterpret_cast<const bf16x4*>(cp), o4;
+                                    if (EPI == EPI_BIAS_GELU) {
+                                        *reinterpret_cast<u32x4*>(g.aux + o) = x.u;
 #pragma unroll
-                                    for (int e = 0; e < 4; e++) o4[e] = (__bf16)((float)old[e] + x.f[e]);
-                                    *reinterpret_cast<bf16x4*>(cp) = o4;
-                                }
-                            }
-                        } else {
-                            const int n = wn0 + pass * 64 + ch * 8;
-                            if (m < g.M && n < g.N) {
-                                const size_t o = (size_t)m * g.ldc + n;
-                                union { u32x4 u; bf16x8 h; } x, y, z;
-                                x.u = raw;
-                                if (EPI == EPI_BIAS_GELU) {
-                                    *reinterpret_cast<u32x4*>(g.aux + o) = x.u;
+                                        for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
+                                        *reinterpret_cast<u32x4*>(g.C + o) = y.u;
+                                    } else if (EPI == EPI_DGELU) {
+                                        z.u = *reinterpret_cast<const u32x4*>(g.aux + o);
 #pragma unroll
-                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                    *reinterpret_cast<u32x4*>(g.C + o) = y.u;
-                                } else if (EPI == EPI_DGELU) {
-                                    z.u = *reinterpret_cast<const u32x4*>(g.aux + o);
-#pragma unroll
-                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)z.h[e]) * (float)x.h[e]);
-                                    *reinterpret_cast<u32x4*>(g.C + o) = y.u;
-                                } else {
-                                    *reinterpret_cast<u32x4*>(g.C + o) = x.u;
+                                        for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)z.h[e]) * (float)x.h[e]);
+                                        *reinterpret_cast<u32x4*>(g.C + o) = y.u;
+                                    } else {
+                                        *reinterpret_cast<u32x4*>(g.C + o) = x.u;
+                                    }
                                 }
                             }
                         }
+                        __builtin_amdgcn_s_waitcnt(0xC07F);          // strip reads done before it is overwritten
+                        __builtin_amdgcn_wave_barrier();
                     }
-                    __builtin_amdgcn_s_waitcnt(0xC07F);          // strip reads done before it is overwritten
-                    __builtin_amdgcn_wave_barrier();
                 }
             }
         }

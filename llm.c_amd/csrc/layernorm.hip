@@ -284,11 +284,11 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
     }
 }
 
-// dweight[c] += sum_blocks partial[b][0][c]; dbias likewise. A workgroup owns 32 columns; its 8 row
-// groups each add every 8th partial in ascending order, then the 8 sub-sums are added in group order:
-// a fixed summation tree, so the result is reproducible, with 8x the memory parallelism of one thread
+// dweight[c] += sum_blocks partial[b][0][c]; dbias likewise. A workgroup owns 32 columns; its 32 row
+// groups each add every 32nd partial in ascending order, then the 32 sub-sums are added in group order:
+// a fixed summation tree, so the result is reproducible, with 32x the memory parallelism of one thread
 // per column.
-constexpr int LNR_COLS = 32, LNR_GROUPS = 8;
+constexpr int LNR_COLS = 32, LNR_GROUPS = 32;
 __global__ void __launch_bounds__(LNR_COLS * LNR_GROUPS)
 ln_backward_reduce_kernel(floatX* __restrict__ dweight, floatX* __restrict__ dbias, const float* __restrict__ partial,
                           int nblocks, int C) {
