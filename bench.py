@@ -93,6 +93,12 @@ def main():
               "use --gpus 1", file=sys.stderr)
         sys.exit(2)
 
+    # the native driver and the reference's CPU trainer print their model headers with printf: send everything
+    # written to file descriptor 1 to stderr until the result line, so stdout carries exactly one JSON line
+    sys.stdout.flush()
+    real_stdout = os.dup(1)
+    os.dup2(2, 1)
+
     import torch
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     pkg = package()
@@ -180,7 +186,11 @@ def main():
     }
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
-    print(json.dumps(out))
+    C.CDLL(None).fflush(None)
+    sys.stdout.flush()
+    os.dup2(real_stdout, 1)
+    os.close(real_stdout)
+    print(json.dumps(out), flush=True)
 
 
 def ctypes_float(x):

@@ -263,7 +263,7 @@ constexpr int BIG_TILE = 256, SMALL_TILE = 128, K_STEP = 64;
 // leading dimensions and N multiples of 8, 16-byte aligned operands, 8-byte aligned bias.
 bool pipelined_ok(const GemmArgs& g) {
     auto al = [](const void* p, uintptr_t a) { return ((uintptr_t)p % a) == 0; };
-    return g.K % PBK == 0 && g.k_per_split % PBK == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 8 == 0 &&
+    return g.K % KGRAN == 0 && g.k_per_split % KGRAN == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 8 == 0 &&
            g.N % 8 == 0 && al(g.A, 16) && al(g.B, 16) && al(g.C, 16) && (!g.bias || al(g.bias, 8)) && (!g.aux || al(g.aux, 16));
 }
 template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
@@ -601,6 +601,17 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         const bool big = tiles_big >= 8;                          // split-K fills the machine when there are few big tiles
         const size_t tiles = big ? tiles_big : tiles_small;
         int splits = (int)max((size_t)1, (size_t)num_cu / tiles);
+        if (tiles > (size_t)num_cu) {
+            // More tiles than CUs: the last round of a persistent launch may be mostly empty (591 tiles on 256 CUs
+            // run as 3 rounds at 77 %). Splitting K by a small factor evens the rounds out; each extra split costs
+            // one fp32 pass over the output, priced here at 2 % of the GEMM.
+            double best = 1e30;
+            for (int s = 1; s <= 4; s++) {
+                const size_t work = tiles * s, rounds = CEIL_DIV(work, (size_t)num_cu);
+                const double cost = (double)(rounds * num_cu) / (double)work + (s > 1 ? 0.02 * s : 0.0);
+                if (cost < best) { best = cost; splits = s; }
+            }
+        }
         const int ksteps = CEIL_DIV(M, K_STEP);
         splits = min(splits, max(1, ksteps / 8));                 // at least 8 K steps per split
         const int steps_per = CEIL_DIV(ksteps, splits);

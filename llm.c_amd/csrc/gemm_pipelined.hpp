@@ -29,6 +29,7 @@
 #pragma once
 #include "common.hpp"
 #include "gelu.hpp"
+#include <type_traits>
 
 namespace gemmk {
 
@@ -57,7 +58,8 @@ struct GemmArgs {
 #if !defined(LLMK_FP32)
 
 constexpr int PBK = 32;                 // K per pipeline block
-constexpr int STAGES = 5;                // ring slots; loads run STAGES-1 K blocks ahead of the math
+constexpr int STAGES = 5;               // ring slots of one K block: two pairs of blocks and a spare for the epilogue
+constexpr int KGRAN = 2 * PBK;          // K (and the K range of a split) must be a multiple of this
 constexpr int LDS_TOTAL = 160 * 1024;
 constexpr int EPI_PITCH = 144;          // bytes per staged output row: 128 + 16
 
@@ -72,10 +74,24 @@ __device__ __forceinline__ void wait_vmcnt() {
 // Workgroup barrier WITHOUT the memory fence of __syncthreads(): the fence would wait for every outstanding
 // direct-to-LDS load (vmcnt(0)) and serialize the pipeline. Visibility of the K block that is about to be
 // read is established by the explicit vmcnt wait each wave does before arriving here.
+template <int DBG = 0>
 __device__ __forceinline__ void barrier_no_fence() {
+    if (DBG & 8) return;
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+}
+
+// Output stores are non-temporal: a tile's output is not read again by this kernel, and a store that allocates in
+// L2 is acknowledged late enough (the waves count stores and loads with one counter) to hold up the next tile's loads.
+template <int DBG = 0, typename T>
+__device__ __forceinline__ void st_out(T* p, T v) {
+    if (DBG & 4096) *p = v; else __builtin_nontemporal_store(v, p);
+}
+// ... except where the next kernel reads a small result straight back (split-K partial sums, weight gradients)
+template <typename T>
+__device__ __forceinline__ void st_cached(T* p, T v) {
+    *p = v;
 }
 
 // tile id -> tile coordinates; consecutive ids walk an 8-row group of tiles column by column
@@ -89,7 +105,7 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int& tm
     tn = in_group / gsz;
 }
 
-template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI, int DBG = 0>   // DBG: measurement ablations (1: no loads, 2: no math)
+template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI, int DBG = 0>   // DBG: measurement ablations (1: no loads, 2: no math, 4: no stores)
 __global__ void __launch_bounds__(WGM * WGN * 64)
 gemm_pipelined_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only builtins below; the host pass only needs the launch stub
@@ -97,6 +113,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
     constexpr int A_STAGE = BM * PBK * 2, B_STAGE = BN * PBK * 2, STAGE = A_STAGE + B_STAGE;
     constexpr int A_CHUNKS = A_STAGE / 1024, B_CHUNKS = B_STAGE / 1024;
+    constexpr int PASSES_OF_EPI = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
     static_assert(STAGES * STAGE <= LDS_TOTAL, "LDS budget");
@@ -105,8 +122,22 @@ gemm_pipelined_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
+    if (DBG & 64) {  // experiment: stagger the workgroups of an XCD over one tile period
+        const int phase = (blockIdx.x >> 3) & 7;
+        for (int i = 0; i < phase; i++) __builtin_amdgcn_s_sleep(100);
+    }
+    if (DBG & 1) {   // ablation without loads: define the LDS contents (32: pseudo-random bits, else zeros)
+        for (int i = tid * 4; i < STAGES * STAGE; i += NT * 4) {
+            unsigned v = (DBG & 32) ? ((squirrel_noise5((uint32_t)i, 17u) & 0x3fff3fffu) | 0x30003000u) : 0u;
+            *reinterpret_cast<unsigned*>(lds + i) = v;
+        }
+        __syncthreads();
+    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // scalar: LDS-DMA destinations must be wave-uniform
     const int wm = wave / WGN, wn = wave % WGN;
+    // The two waves that share a SIMD (w and w + NW/2) request their share of a K block at different points of
+    // the block's math, so that a wave held up at the memory pipeline's entrance always has a partner issuing MFMAs.
+    const bool late = (DBG & 2048) ? false : wave >= NW / 2;
     const int idx = lane & 31, half = lane >> 5;
     const int tiles_m = CEIL_DIV(g.M, BM), tiles_n = CEIL_DIV(g.N, BN);
     const int num_tiles = tiles_m * tiles_n;
@@ -142,7 +173,11 @@ gemm_pipelined_kernel(GemmArgs g) {
             constexpr int RA = BM, RB = BN;
             const int R = isA ? RA : RB;
             lds_dst[i] = (isA ? 0 : A_STAGE) + cc * 1024;
-            if (!trans) {
+            if (!trans && (DBG & 256)) {   // experiment (loads only): full 128-byte lines per row
+                const int row = cc * 8 + (lane >> 3), p = lane & 7;
+                gp[i] = base + (size_t)min(r0 + row, rmax - 1) * ld + kbeg + p * 8;
+                kstep[i] = (size_t)128 * ld;
+            } else if (!trans) {
                 const int row = cc * 16 + (lane >> 2), p = lane & 3;
                 const int c = p ^ ((row >> 2) & 3);
                 const int grow = min(r0 + row, rmax - 1);
@@ -151,7 +186,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             } else {
                 const int byte = cc * 1024 + lane * 16;
                 const int krow = byte / (R * 2), p = (byte % (R * 2)) >> 4;
-                const int cn = p ^ (4 * (krow & 3));
+                const int cn = (DBG & 16384) ? p : p ^ (4 * (krow & 3));
                 int col = r0 + cn * 8;
                 if (col >= rmax) col = r0;
                 gp[i] = base + (size_t)(kbeg + krow) * ld + col;
@@ -159,12 +194,16 @@ gemm_pipelined_kernel(GemmArgs g) {
             }
         }
     };
-    auto issue = [&](int kb, int slot) {
-        char* stage = lds + slot * STAGE;
+    // two consecutive K blocks at once, the two 64-byte halves of every 128-byte line requested back to back
+    auto issue2 = [&](int kb, int slot0, int slot1) {
+        char* stage0 = lds + slot0 * STAGE;
+        char* stage1 = lds + slot1 * STAGE;
         if (DBG & 1) return;
 #pragma unroll
-        for (int i = 0; i < CPW; i++)
-            __builtin_amdgcn_global_load_lds(gp[i] + (size_t)kb * kstep[i], (lds_void_ptr)(stage + lds_dst[i]), 16, 0, 0);
+        for (int i = 0; i < CPW; i++) {
+            __builtin_amdgcn_global_load_lds(gp[i] + (size_t)kb * kstep[i], (lds_void_ptr)(stage0 + lds_dst[i]), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds(gp[i] + (size_t)(kb + 1) * kstep[i], (lds_void_ptr)(stage1 + lds_dst[i]), 16, 0, 0);
+        }
     };
 
     // --- MFMA operand reads ----------------------------------------------------------------------
@@ -191,7 +230,60 @@ gemm_pipelined_kernel(GemmArgs g) {
         return u.v;
     };
 
+    // fragments of one 16-wide K step
+    auto read_frags = [&](const char* sa, int s, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
+        if (DBG & 16) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
+#pragma unroll
+            for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
+            return;
+        }
+        const char* sb = sa + A_STAGE;
+#pragma unroll
+        for (int i = 0; i < TM; i++) fa[i] = A_T ? frag_t(sa, BM * 2, wm * WTM + i * 32, s) : frag_k(sa, wm * WTM + i * 32, s);
+        if (DBG & 512) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
+            return;
+        }
+#pragma unroll
+        for (int j = 0; j < TN; j++) fb[j] = B_T ? frag_t(sb, BN * 2, wn * WTN + j * 32, s) : frag_k(sb, wn * WTN + j * 32, s);
+    };
+    // Hand-issued (transposing) reads have to be awaited by hand. LDS operations return in order, so "at most
+    // YOUNGER operations outstanding" means these operands have arrived when YOUNGER hand-issued reads were
+    // requested after them (compiler-issued reads in between only make the wait longer). The operands are tied
+    // to the wait so that nothing that uses them moves above it.
+    constexpr int TR_READS = (A_T ? 2 * TM : 0) + (B_T ? 2 * TN : 0);       // hand-issued reads per 16-wide step
+    auto await_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], auto younger) {
+        constexpr int Y = decltype(younger)::value;
+        if (A_T) {
+#pragma unroll
+            for (int i = 0; i < TM; i++) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(fa[i]) : "n"(Y));
+        }
+        if (B_T) {
+#pragma unroll
+            for (int j = 0; j < TN; j++) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(fb[j]) : "n"(Y));
+        }
+    };
+    using Younger = std::integral_constant<int, TR_READS>;
+    using NoneYounger = std::integral_constant<int, 0>;
     f32x16 acc[TM][TN];
+    auto mma = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
+        if (DBG & 2) return;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)   // swapped operands: acc[i][j] = D^T block, rows = n, cols = m
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+    };
+    // Waiting for loads: vector-memory operations retire in issue order, so "at most N outstanding" means that
+    // everything but the N youngest has landed. The pairs of a tile are requested one at a time, so the only
+    // younger operations a wait ever has to allow are the second pair of the tile's prologue and the previous
+    // tile's output stores (NS_EPI per wave when every lane stored, which holds for interior tiles).
+    constexpr int NS_EPI = TM * PASSES_OF_EPI * 4 * (EPI == EPI_BIAS_GELU ? 2 : 1);
+    static_assert(2 * CPW + NS_EPI <= 63, "vmcnt is a 6-bit counter");
+
     int ring = 0;                       // ring slot that holds K block 0 of the current work item
     int it = 0;
     int w = work_id(0);
@@ -202,9 +294,43 @@ gemm_pipelined_kernel(GemmArgs g) {
     int kbeg = split * g.k_per_split;
     int nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
     setup_loads(tile_m * BM, tile_n * BN, kbeg);
+    issue2(0, ring % STAGES, (ring + 1) % STAGES);
+    if (nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
+    bool st_young = false;              // the previous epilogue's stores are all issued and counted
+
+    // Epilogues that read global memory (the pre-GELU activations, the old weight gradient) request it while the
+    // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
+    constexpr bool F32OUT = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
+    constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
+    constexpr bool EPI_READS = (EPI == EPI_DGELU || EPI == EPI_ACCUM);
+    u32x4 pre_aux[EPI == EPI_DGELU ? TM : 1][2][2];
+    bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
+    auto prefetch_epilogue = [&](int tm0, int tn0) {
+        if (!EPI_READS || (DBG & 4)) return;
+        const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
 #pragma unroll
-    for (int j = 0; j < STAGES - 1; j++)
-        if (j < nkb) issue(j, (ring + j) % STAGES);
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int pass = 0; pass < PASSES; pass++)
+#pragma unroll
+                for (int hsel = 0; hsel < 2; hsel++)
+#pragma unroll
+                    for (int t = 0; t < 2; t++) {
+                        const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                        const int m = wm0 + i * 32 + hsel * 16 + row;
+                        if (EPI == EPI_DGELU) {
+                            const int n = wn0 + pass * 64 + ch * 8;
+                            if (m < g.M && n < g.N) pre_aux[i][hsel][t] = *reinterpret_cast<const u32x4*>(g.aux + (size_t)m * g.ldc + n);
+                        } else {
+                            const int n = wn0 + pass * 32 + ch * 4;
+                            if (m < g.M && n < g.N) pre_old[i][pass][hsel][t] = *reinterpret_cast<const bf16x4*>(g.C + (size_t)m * g.ldc + n);
+                        }
+                    }
+    };
+
+    long long tc[8] = {0, 0, 0, 0, 0, 0, 0, 0};        // DBG & 128: cycle counts by phase (wave 0)
+    auto now = [&]() -> long long { return (DBG & 128) ? (long long)__builtin_readcyclecounter() : 0; };
+    const long long t_kernel = now();
 
     while (true) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -215,44 +341,63 @@ gemm_pipelined_kernel(GemmArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-        // ---- K loop -----------------------------------------------------------------------------
-        for (int kb = 0; kb < nkb; kb++) {
-            const int ahead = min(STAGES - 2, nkb - 1 - kb);      // younger blocks that may stay in flight
-            if (ahead >= 3) wait_vmcnt<3 * CPW>();
-            else if (ahead == 2) wait_vmcnt<2 * CPW>();
-            else if (ahead == 1) wait_vmcnt<CPW>();
-            else wait_vmcnt<0>();
-            barrier_no_fence();                                   // block kb landed for everyone; slot of kb-1 is free
-            if (kb + STAGES - 1 < nkb) issue(kb + STAGES - 1, (ring + kb + STAGES - 1) % STAGES);
-            const char* sa = lds + ((ring + kb) % STAGES) * STAGE;
-            const char* sb = sa + A_STAGE;
-#pragma unroll
-            for (int s = 0; s < ((DBG & 2) ? 0 : PBK / 16); s++) {
-                bf16x8 fa[TM], fb[TN];
-#pragma unroll
-                for (int i = 0; i < TM; i++) fa[i] = A_T ? frag_t(sa, BM * 2, wm * WTM + i * 32, s) : frag_k(sa, wm * WTM + i * 32, s);
-#pragma unroll
-                for (int j = 0; j < TN; j++) fb[j] = B_T ? frag_t(sb, BN * 2, wn * WTN + j * 32, s) : frag_k(sb, wn * WTN + j * 32, s);
-                if (A_T || B_T) {      // hand-issued reads: wait for LDS, with the operands tied to the wait so nothing moves above it
-                    if (A_T) {
-#pragma unroll
-                        for (int i = 0; i < TM; i++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fa[i]));
-                    }
-                    if (B_T) {
-#pragma unroll
-                        for (int j = 0; j < TN; j++) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(fb[j]));
-                    }
-                }
-#pragma unroll
-                for (int i = 0; i < TM; i++)
-#pragma unroll
-                    for (int j = 0; j < TN; j++)   // swapped operands: acc[i][j] = D^T block, rows = n, cols = m
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
-            }
+        // ---- K loop over pairs of K blocks (one barrier per 64 of K), software-pipelined: the operands of the
+        // next 16-wide step (and the barrier that publishes the next pair) are requested while the matrix cores
+        // work on the current step. Pair p lives in ring slots 2p and 2p+1 (mod STAGES); while pair p is
+        // multiplied, pair p+1 is in flight and the fifth slot is spare (the epilogue's).
+        bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+        const int npairs = nkb >> 1;                              // the host guarantees an even number of K blocks
+        auto slot_of = [&](int kb) -> const char* { return lds + ((ring + kb) % STAGES) * STAGE; };
+        auto issue_pair = [&](int q) { issue2(2 * q, (ring + 2 * q) % STAGES, (ring + 2 * q + 1) % STAGES); };
+        long long ta = now();
+        if (npairs >= 2) { if (st_young) wait_vmcnt<2 * CPW + NS_EPI>(); else wait_vmcnt<2 * CPW>(); }
+        else wait_vmcnt<0>();
+        barrier_no_fence<DBG>();                                  // pair 0 landed for everyone
+        long long tb = now();
+        tc[0] += tb - ta;
+        const long long t_loop = tb;
+        read_frags(slot_of(0), 0, fa0, fb0);
+        for (int p = 0; p < npairs - 1; p++) {
+            read_frags(slot_of(2 * p), 1, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0);
+            if (late && p >= 1) issue_pair(p + 1);
+            read_frags(slot_of(2 * p + 1), 0, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1);
+            read_frags(slot_of(2 * p + 1), 1, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0);
+            __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading pair p
+            ta = now();
+            if (p == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // pair p+1 has landed (for this wave's share)
+            if (DBG & 128) { tb = now(); tc[6] += tb - ta; }
+            barrier_no_fence<DBG>();                              // ... and for everyone; the slots of pair p are free
+            if (DBG & 128) { tb = now(); tc[2] += tb - ta; }
+            if (!late && p + 2 < npairs) issue_pair(p + 2);
+            read_frags(slot_of(2 * p + 2), 0, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1);
         }
+        {
+            const int p = npairs - 1;
+            prefetch_epilogue(m0, n0);
+            read_frags(slot_of(2 * p), 1, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0);
+            read_frags(slot_of(2 * p + 1), 0, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1);
+            read_frags(slot_of(2 * p + 1), 1, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0);
+            await_frags(fa1, fb1, NoneYounger{});
+            mma(fa1, fb1);
+        }
+        if (DBG & 128) { ta = now(); tc[3] += ta - t_loop; }
 
         // ---- request the next work item's first K blocks, then run the epilogue under them --------
-        barrier_no_fence();                                       // every wave is done reading the ring
+        barrier_no_fence<DBG>();                                       // every wave is done reading the ring
         const int ring_free = (ring + nkb) % STAGES;              // slot the epilogue may use
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
         it++;
@@ -266,9 +411,8 @@ gemm_pipelined_kernel(GemmArgs g) {
             next_nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
             setup_loads(tile_m * BM, tile_n * BN, kbeg);
             ring = (ring_free + 1) % STAGES;
-#pragma unroll
-            for (int j = 0; j < STAGES - 1; j++)
-                if (j < next_nkb) issue(j, (ring + j) % STAGES);
+            issue2(0, ring % STAGES, (ring + 1) % STAGES);
+            if (!(DBG & 8192) && next_nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
         }
 
         // ---- epilogue ---------------------------------------------------------------------------------
@@ -279,8 +423,6 @@ gemm_pipelined_kernel(GemmArgs g) {
             static_assert(NW * STRIP <= STAGE, "all strips must fit in one ring slot");
             char* strip = lds + ring_free * STAGE + wave * STRIP;
             const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
-            constexpr bool F32OUT = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
-            constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
             constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
 #pragma unroll
             for (int i = 0; i < TM; i++) {
@@ -332,37 +474,37 @@ gemm_pipelined_kernel(GemmArgs g) {
                             u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * EPI_PITCH + ch * 16);
                             if (F32OUT) {
                                 const int n = wn0 + pass * 32 + ch * 4;
-                                if (m < g.M && n < g.N) {
+                                if (m < g.M && n < g.N && !(DBG & 4)) {
                                     if (EPI == EPI_PARTIAL) {
-                                        *reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n) = raw;
+                                        st_cached(reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n), raw);
                                     } else {
                                         union { u32x4 u; f32x4 f; } x;
                                         x.u = raw;
                                         floatX* cp = g.C + (size_t)m * g.ldc + n;
-                                        bf16x4 old = *reinterpret_cast<const bf16x4*>(cp), o4;
+                                        bf16x4 old = pre_old[EPI == EPI_ACCUM ? i : 0][EPI == EPI_ACCUM ? pass : 0][hsel][t], o4;
 #pragma unroll
                                         for (int e = 0; e < 4; e++) o4[e] = (__bf16)((float)old[e] + x.f[e]);
-                                        *reinterpret_cast<bf16x4*>(cp) = o4;
+                                        st_cached(reinterpret_cast<bf16x4*>(cp), o4);
                                     }
                                 }
                             } else {
                                 const int n = wn0 + pass * 64 + ch * 8;
-                                if (m < g.M && n < g.N) {
+                                if (m < g.M && n < g.N && !(DBG & 4)) {
                                     const size_t o = (size_t)m * g.ldc + n;
                                     union { u32x4 u; bf16x8 h; } x, y, z;
                                     x.u = raw;
                                     if (EPI == EPI_BIAS_GELU) {
-                                        *reinterpret_cast<u32x4*>(g.aux + o) = x.u;
+                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.aux + o), x.u);
 #pragma unroll
                                         for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                        *reinterpret_cast<u32x4*>(g.C + o) = y.u;
+                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                     } else if (EPI == EPI_DGELU) {
-                                        z.u = *reinterpret_cast<const u32x4*>(g.aux + o);
+                                        z.u = pre_aux[EPI == EPI_DGELU ? i : 0][hsel][t];
 #pragma unroll
                                         for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)z.h[e]) * (float)x.h[e]);
-                                        *reinterpret_cast<u32x4*>(g.C + o) = y.u;
+                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                     } else {
-                                        *reinterpret_cast<u32x4*>(g.C + o) = x.u;
+                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), x.u);
                                     }
                                 }
                             }
@@ -373,8 +515,16 @@ gemm_pipelined_kernel(GemmArgs g) {
                 }
             }
         }
+        if ((DBG & 8192) && have_next && next_nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
+        if (DBG & 128) { tb = now(); tc[4] += tb - ta; }
         if (!have_next) break;
+        st_young = (DBG & 8192) ? false : cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
         nkb = next_nkb;
+    }
+    if ((DBG & 128) && lane == 0) {
+        tc[5] = now() - t_kernel;
+        long long* o = reinterpret_cast<long long*>(g.partial) + (blockIdx.x * NW + wave) * 8;
+        for (int i = 0; i < 8; i++) o[i] = tc[i];
     }
 #endif  // __HIP_DEVICE_COMPILE__
 }
