@@ -56,6 +56,8 @@ void llmk_clear_error(void);
  * every kernel launch of this library is bracketed by HIP events on its stream; the report aggregates
  * by kernel family: number of launches, total milliseconds, algorithmic flops and algorithmic bytes. */
 void llmk_profile_enable(int on);
+/* NULL or "": time every family; otherwise only launches of the named family are bracketed by events */
+void llmk_profile_only(const char* family);
 void llmk_profile_reset(void);
 int llmk_profile_count(void);
 void llmk_profile_get(int i, char* name64, int* calls, double* ms, double* flops, double* bytes);

@@ -47,13 +47,13 @@ void* workspace(size_t bytes);
 // marks the same spots with NVTX ranges and post-processes an ncu run (llmc/cuda_common.h:115-124,
 // profile_gpt2cu.py); here the library can time its own launches and report time, algorithmic
 // flops and algorithmic bytes per kernel family.
-bool profiling();
+bool profiling(const char* name);
 void prof_begin(const char* name, double flops, double bytes, hipStream_t st);
 void prof_end(hipStream_t st);
 struct ProfScope {
     hipStream_t st;
     bool on;
-    ProfScope(const char* name, double flops, double bytes, hipStream_t s) : st(s), on(profiling()) {
+    ProfScope(const char* name, double flops, double bytes, hipStream_t s) : st(s), on(profiling(name)) {
         if (on) prof_begin(name, flops, bytes, st);
     }
     ~ProfScope() { if (on) prof_end(st); }

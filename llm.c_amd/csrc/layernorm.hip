@@ -183,49 +183,56 @@ residual_kernel(floatX* __restrict__ out, const floatX* __restrict__ a, const fl
 // At the end the 4 waves of a workgroup are added in wave order through LDS and the workgroup's
 // partial goes to scratch[block][2][C]; a second kernel adds the partials in block order, so
 // the result does not depend on scheduling (no atomics).
+// One workgroup per CU, as many waves as the accumulators leave room for: 12 (three per SIMD) up to NV = 2, where the
+// kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8, then 4 beyond.
+constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 4 ? 8 : 4; }
 template <int NV>
-__global__ void __launch_bounds__(LN_BLOCK)
+__global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : 1)
 ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
                    const floatX* __restrict__ inp, const floatX* __restrict__ weight,
                    const float* __restrict__ mean, const float* __restrict__ rstd, int N, int C) {
-    extern __shared__ float lds[];   // [LN_WAVES-1][2][C]
+    constexpr int LNB_WAVES = lnb_waves(NV);
+    extern __shared__ float lds[];   // [LNB_WAVES-1][2][C]
     const int lane = threadIdx.x & 63;
     const int wid = threadIdx.x >> 6;
-    const int wave = blockIdx.x * LN_WAVES + wid;
-    const int nwaves = gridDim.x * LN_WAVES;
+    const int wave = blockIdx.x * LNB_WAVES + wid;
+    const int nwaves = gridDim.x * LNB_WAVES;
     const int nvec = C / VN;
     const float invC = 1.0f / (float)C;
 
-    float w[NV][VN], dw[NV][VN], db[NV][VN];
+    vecX w[NV];                          // packed: the fp32 copy would cost 8 more registers per vector
+    float dw[NV][VN], db[NV][VN];
 #pragma unroll
     for (int i = 0; i < NV; i++) {
         int v = lane + i * 64;
-        vecX wv;
-        if (v < nvec) wv = ld_vec(weight + (size_t)v * VN);
+        if (v < nvec) w[i] = ld_vec(weight + (size_t)v * VN);
 #pragma unroll
-        for (int k = 0; k < VN; k++) { w[i][k] = v < nvec ? to_f32(wv[k]) : 0.f; dw[i][k] = 0.f; db[i][k] = 0.f; }
+        for (int k = 0; k < VN; k++) { dw[i][k] = 0.f; db[i][k] = 0.f; }
     }
 
-    for (int row = wave; row < N; row += nwaves) {
+    // Two rows are in flight per wave: the loads of the next row are issued before the current row is reduced,
+    // which doubles the bytes each CU keeps in flight at the occupancy the accumulators allow.
+    auto load_row = [&](int row, vecX (&g)[NV], vecX (&x)[NV], vecX (&di)[NV]) {
         const size_t base = (size_t)row * C;
-        vecX g[NV], x[NV], di[NV];
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             int v = lane + i * 64;
             if (v < nvec) {
                 g[i] = ld_vec_nt(dout + base + (size_t)v * VN);
                 x[i] = ld_vec_nt(inp + base + (size_t)v * VN);
-                di[i] = ld_vec(dinp + base + (size_t)v * VN);
+                di[i] = ld_vec_nt(dinp + base + (size_t)v * VN);
             }
         }
-        const float m = mean[row], r = rstd[row];
+    };
+    auto process_row = [&](int row, float m, float r, const vecX (&g)[NV], const vecX (&x)[NV], const vecX (&di)[NV]) {
+        const size_t base = (size_t)row * C;
         float a = 0.f, bsum = 0.f;
 #pragma unroll
         for (int i = 0; i < NV; i++)
             if (lane + i * 64 < nvec) {
 #pragma unroll
                 for (int k = 0; k < VN; k++) {
-                    float nh = (to_f32(x[i][k]) - m) * r, dn = w[i][k] * to_f32(g[i][k]);
+                    float nh = (to_f32(x[i][k]) - m) * r, dn = to_f32(w[i][k]) * to_f32(g[i][k]);
                     a += dn;
                     bsum += dn * nh;
                 }
@@ -240,13 +247,29 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
 #pragma unroll
                 for (int k = 0; k < VN; k++) {
                     float gk = to_f32(g[i][k]);
-                    float nh = (to_f32(x[i][k]) - m) * r, dn = w[i][k] * gk;
+                    float nh = (to_f32(x[i][k]) - m) * r, dn = to_f32(w[i][k]) * gk;
                     db[i][k] += gk;
                     dw[i][k] += nh * gk;
                     o[k] = from_f32<floatX>(to_f32(di[i][k]) + (dn - a - nh * bsum) * r);
                 }
                 st_vec(dinp + base + (size_t)v * VN, o);
             }
+        }
+    };
+    {
+        vecX g0[NV], x0[NV], d0[NV], g1[NV], x1[NV], d1[NV];
+        int row = wave;
+        float m0 = 0.f, r0 = 0.f, m1 = 0.f, r1 = 0.f;
+        if (row < N) { load_row(row, g0, x0, d0); m0 = mean[row]; r0 = rstd[row]; }
+        while (row < N) {
+            const int row1 = row + nwaves;
+            if (row1 < N) { load_row(row1, g1, x1, d1); m1 = mean[row1]; r1 = rstd[row1]; }
+            process_row(row, m0, r0, g0, x0, d0);
+            if (row1 >= N) break;
+            const int row2 = row1 + nwaves;
+            if (row2 < N) { load_row(row2, g0, x0, d0); m0 = mean[row2]; r0 = rstd[row2]; }
+            process_row(row1, m1, r1, g1, x1, d1);
+            row = row2;
         }
     }
 
@@ -272,7 +295,7 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
 #pragma unroll
                 for (int k = 0; k < VN; k++) {
                     float sw = dw[i][k], sb = db[i][k];
-                    for (int o = 0; o < LN_WAVES - 1; o++) {
+                    for (int o = 0; o < LNB_WAVES - 1; o++) {
                         sw += lds[(size_t)o * 2 * C + v * VN + k];
                         sb += lds[(size_t)o * 2 * C + C + v * VN + k];
                     }
@@ -309,7 +332,7 @@ ln_backward_reduce_kernel(floatX* __restrict__ dweight, floatX* __restrict__ dbi
     }
 }
 
-int ln_backward_blocks() { return llmk::device_info().num_cu * 4; }
+int ln_backward_blocks() { return llmk::device_info().num_cu; }
 
 }  // namespace
 
@@ -357,16 +380,23 @@ void llmk_layernorm_backward(void* dinp, void* dweight, void* dbias, float* scra
     const int N = B * T;
     if (N == 0) return;
     hipStream_t st = (hipStream_t)stream;
-    int blocks = min(ln_backward_blocks(), CEIL_DIV(N, LN_WAVES));
-    size_t smem = (size_t)(LN_WAVES - 1) * 2 * C * sizeof(float);
+    const int waves = lnb_waves(nv);
+    const int blocks = min(ln_backward_blocks(), CEIL_DIV(N, waves));
+    const size_t smem = (size_t)(waves - 1) * 2 * C * sizeof(float);
     {
     llmk::ProfScope prof("layernorm_backward", 0, 4.0 * N * C * sizeof(floatX) + 2.0 * N * sizeof(float), st);
 #define LNB_CASE(K)                                                                                          \
-    case K:                                                                                                  \
-        ln_backward_kernel<K><<<blocks, LN_BLOCK, smem, st>>>((floatX*)dinp, scratch, (const floatX*)dout,   \
+    case K: {                                                                                                \
+        static bool attr_set = false;                                                                        \
+        if (!attr_set) {                                                                                     \
+            HIP_CHECK(hipFuncSetAttribute((const void*)ln_backward_kernel<K>,                                \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));          \
+            attr_set = true;                                                                                 \
+        }                                                                                                    \
+        ln_backward_kernel<K><<<blocks, lnb_waves(K) * 64, smem, st>>>((floatX*)dinp, scratch, (const floatX*)dout, \
                                                               (const floatX*)inp, (const floatX*)weight,    \
                                                               mean, rstd, N, C);                             \
-        break;
+        break; }
     switch (nv) { LNB_CASE(1) LNB_CASE(2) LNB_CASE(3) LNB_CASE(4) LNB_CASE(5) LNB_CASE(6) LNB_CASE(7) LNB_CASE(8) }
 #undef LNB_CASE
     LAUNCH_CHECK();

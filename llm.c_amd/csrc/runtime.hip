@@ -70,7 +70,8 @@ static std::vector<ProfRec> g_prof_recs;
 static std::vector<hipEvent_t> g_event_pool;
 static std::vector<ProfAgg> g_prof_agg;
 
-bool profiling() { return g_prof_on; }
+static std::string g_prof_only;   // when not empty: only this kernel family is timed
+bool profiling(const char* name) { return g_prof_on && (g_prof_only.empty() || g_prof_only == name); }
 static hipEvent_t take_event() {
     if (!g_event_pool.empty()) { hipEvent_t e = g_event_pool.back(); g_event_pool.pop_back(); return e; }
     hipEvent_t e;
@@ -106,6 +107,7 @@ static void prof_collect() {
 extern "C" {
 
 void llmk_profile_enable(int on) { llmk::prof_collect(); llmk::g_prof_on = on != 0; }
+void llmk_profile_only(const char* family) { llmk::g_prof_only = family ? family : ""; }
 void llmk_profile_reset(void) { llmk::prof_collect(); llmk::g_prof_agg.clear(); }
 int llmk_profile_count(void) { llmk::prof_collect(); return (int)llmk::g_prof_agg.size(); }
 void llmk_profile_get(int i, char* name64, int* calls, double* ms, double* flops, double* bytes) {
