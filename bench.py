@@ -87,6 +87,9 @@ def main():
     ap.add_argument("--gelu-fusion", type=int, default=2)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first launch one copy kernel of known size (128 MiB read, 256 MiB written): the yardstick for "
+                         "scaling FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs the training step on ONE GPU only (no collectives are part of it); "
@@ -117,6 +120,14 @@ def main():
     stream = rng.randint(0, V, size=B * T + 1).astype(np.int32)    # uint16-range tokens, targets = inputs shifted by one
     inp, tgt = np.ascontiguousarray(stream[:-1]), np.ascontiguousarray(stream[1:])
     ip, tp = inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p)
+
+    if args.calibrate_copy:
+        n = 64 * 1024 * 1024
+        src = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+        dst = torch.empty(n, dtype=torch.float32, device="cuda")
+        L.llmk_copy_and_cast_to_f32(dst.data_ptr(), src.data_ptr(), n, 0, 0, 1, None)
+        torch.cuda.synchronize()
+        del src, dst
 
     def step(t):
         L.gpt2_forward(h, ip, B, T)

@@ -279,7 +279,7 @@ void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
     }
     g.splits = splits;
     const int work = CEIL_DIV(g.M, BM) * CEIL_DIV(g.N, BN) * splits;
-    const int grid = min(work, llmk::device_info().num_cu);
+    const int grid = min((work + 7) & ~7, llmk::device_info().num_cu & ~7);   // a multiple of 8: one share per XCD
     kern<<<grid, NW * 64, SMEM, st>>>(g);
     LAUNCH_CHECK();
 }

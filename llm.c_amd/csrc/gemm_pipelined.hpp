@@ -144,16 +144,28 @@ gemm_pipelined_kernel(GemmArgs g) {
     const int num_work = num_tiles * g.splits;
 
     // --- this workgroup's share of the work list ---------------------------------------------
-    // Workgroups are dispatched round-robin over the 8 XCDs; give XCD x the ids [32x, 32x+32) of
-    // every round of 256 so that its CUs share operand panels in its L2.
+    // Workgroups are dispatched round-robin over the 8 XCDs, each with its own L2 (the host launches a multiple
+    // of 8). Without split-K and with enough row panels, XCD x owns the row panels [tiles_m*x/8, tiles_m*(x+1)/8)
+    // outright and its CUs walk them together, 8 panels by all columns at a time: the streamed operand (A) then
+    // crosses HBM once. Otherwise XCD x takes the ids [x*G/8, (x+1)*G/8) of every round, so that a split's tiles
+    // (which share their K range of both operands) sit on one XCD.
     const int G = gridDim.x;
-    auto work_id = [&](int it) -> int {
-        int w = it * G + blockIdx.x;
-        if ((G & 7) == 0) {
-            const int per = G >> 3;
-            w = it * G + (blockIdx.x & 7) * per + (blockIdx.x >> 3);
+    auto work_item = [&](int it, int& tm, int& tn, int& sp) -> bool {
+        const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, per_x = G >> 3;
+        if (!(DBG & 65536) && g.splits == 1 && tiles_m >= 64) {
+            const int r0 = (tiles_m * xcd) >> 3, rows = ((tiles_m * (xcd + 1)) >> 3) - r0;
+            const int q = it * per_x + local;
+            if (q >= rows * tiles_n) return false;
+            tile_of(q, rows, tiles_n, tm, tn);
+            tm += r0;
+            sp = 0;
+            return true;
         }
-        return w;
+        const int w = it * G + xcd * per_x + local;
+        if (w >= num_work) return false;
+        tile_of(w % num_tiles, tiles_m, tiles_n, tm, tn);
+        sp = w / num_tiles;
+        return true;
     };
 
     // --- per-thread load descriptors -----------------------------------------------------------
@@ -286,11 +298,8 @@ gemm_pipelined_kernel(GemmArgs g) {
 
     int ring = 0;                       // ring slot that holds K block 0 of the current work item
     int it = 0;
-    int w = work_id(0);
-    if (w >= num_work) return;
-    int tile_m, tile_n;
-    tile_of(w % num_tiles, tiles_m, tiles_n, tile_m, tile_n);
-    int split = w / num_tiles;
+    int tile_m, tile_n, split;
+    if (!work_item(0, tile_m, tile_n, split)) return;
     int kbeg = split * g.k_per_split;
     int nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
     setup_loads(tile_m * BM, tile_n * BN, kbeg);
@@ -401,12 +410,9 @@ gemm_pipelined_kernel(GemmArgs g) {
         const int ring_free = (ring + nkb) % STAGES;              // slot the epilogue may use
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
         it++;
-        w = work_id(it);
-        const bool have_next = w < num_work;
+        const bool have_next = work_item(it, tile_m, tile_n, split);
         int next_nkb = 0;
         if (have_next) {
-            tile_of(w % num_tiles, tiles_m, tiles_n, tile_m, tile_n);
-            split = w / num_tiles;
             kbeg = split * g.k_per_split;
             next_nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
             setup_loads(tile_m * BM, tile_n * BN, kbeg);
