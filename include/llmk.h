@@ -122,6 +122,14 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                           const void* pre_gelu, int gelu_fusion);
 size_t llmk_matmul_backward_bias_scratch_floats(int OC);
 
+/* gelu_backward_inplace (llmc/gelu.cuh:59) and the bias gradient of matmul_backward (llmc/matmul.cuh:251-266) in
+ * one pass over (B*T, OC): d_in_out *= gelu'(inp), then dbias[OC] += column sums of the result. Same values as
+ * llmk_gelu_backward_inplace followed by llmk_matmul_backward's bias step (bit for bit in the bf16 library, to
+ * the rounding of one fused multiply-add in the fp32 library); the caller then passes dbias = NULL to
+ * llmk_matmul_backward. dbias_buffer: llmk_matmul_backward_bias_scratch_floats(OC) floats. */
+void llmk_gelu_backward_bias(void* d_in_out, const void* inp, void* dbias, float* dbias_buffer, int B, int T, int OC,
+                             void* stream);
+
 /* ---- attention (llmc/cudnn_att.cpp; the flash path the reference takes with ENABLE_CUDNN) -- */
 
 /* attention_forward_cudnn, llmc/cudnn_att.cpp:222. Causal softmax(Q K^T / sqrt(hs)) V.

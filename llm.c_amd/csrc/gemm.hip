@@ -269,8 +269,7 @@ bool pipelined_ok(const GemmArgs& g) {
 template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
 void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
     constexpr int NW = WGM * WGN;
-    constexpr int STAGE = (BM + BN) * PBK * 2;
-    constexpr int SMEM = STAGES * STAGE;
+    constexpr int SMEM = gemmk::smem_bytes(BM, BN, NW);
     auto kern = gemm_pipelined_kernel<BM, BN, WGM, WGN, A_T, B_T, EPI>;
     static bool attr_set = false;
     if (!attr_set) {
@@ -446,9 +445,12 @@ splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, 
 // four row loads in flight. grid.y splits the rows so that ~2 workgroups per CU are resident; their partial sums
 // go to the caller's fp32 scratch and are added in a fixed order by a second, tiny kernel (no atomics).
 constexpr int VN = vecX::N;
+// DGELU: dout is first multiplied in place by gelu'(pre) (rounded to the storage type, and it is the rounded value
+// that is summed, so the result equals gelu_backward_inplace followed by the plain reduction).
 constexpr int BG_COLV = 32, BG_ROWL = 8, BG_UNROLL = 4;
+template <bool DGELU>
 __global__ void __launch_bounds__(256)
-bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, int N, int OC) {
+bias_grad_kernel(float* __restrict__ partial, floatX* __restrict__ dout, const floatX* __restrict__ pre, int N, int OC) {
     __shared__ float red[BG_ROWL][BG_COLV * VN + 1];
     const int cv = threadIdx.x % BG_COLV, rl = threadIdx.x / BG_COLV;
     const int col = (blockIdx.x * BG_COLV + cv) * VN;
@@ -459,16 +461,31 @@ bias_grad_kernel(float* __restrict__ partial, const floatX* __restrict__ dout, i
         const int rstep = gridDim.y * BG_ROWL;
         int r = blockIdx.y * BG_ROWL + rl;
         for (; r + (BG_UNROLL - 1) * rstep < N; r += BG_UNROLL * rstep) {
-            vecX d[BG_UNROLL];
+            vecX d[BG_UNROLL], x[BG_UNROLL];
 #pragma unroll
-            for (int u = 0; u < BG_UNROLL; u++) d[u] = ld_vec_nt(dout + (size_t)(r + u * rstep) * OC + col);
+            for (int u = 0; u < BG_UNROLL; u++) {
+                d[u] = ld_vec_nt(dout + (size_t)(r + u * rstep) * OC + col);
+                if (DGELU) x[u] = ld_vec_nt(pre + (size_t)(r + u * rstep) * OC + col);
+            }
 #pragma unroll
-            for (int u = 0; u < BG_UNROLL; u++)
+            for (int u = 0; u < BG_UNROLL; u++) {
+                if (DGELU) {
+#pragma unroll
+                    for (int k = 0; k < VN; k++) d[u][k] = from_f32<floatX>(gelu_grad_f(to_f32(x[u][k])) * to_f32(d[u][k]));
+                    st_vec(dout + (size_t)(r + u * rstep) * OC + col, d[u]);
+                }
 #pragma unroll
                 for (int k = 0; k < VN; k++) acc[k] += to_f32(d[u][k]);
+            }
         }
         for (; r < N; r += rstep) {
             vecX d = ld_vec_nt(dout + (size_t)r * OC + col);
+            if (DGELU) {
+                vecX x = ld_vec_nt(pre + (size_t)r * OC + col);
+#pragma unroll
+                for (int k = 0; k < VN; k++) d[k] = from_f32<floatX>(gelu_grad_f(to_f32(x[k])) * to_f32(d[k]));
+                st_vec(dout + (size_t)r * OC + col, d);
+            }
 #pragma unroll
             for (int k = 0; k < VN; k++) acc[k] += to_f32(d[k]);
         }
@@ -546,6 +563,22 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
     }
 }
 
+void llmk_gelu_backward_bias(void* d_in_out, const void* inp, void* dbias, float* dbias_buffer, int B, int T, int OC,
+                             void* stream) {
+    if (llmk::failed()) return;
+    const int M = B * T;
+    LLMK_REQUIRE(OC > 0 && OC % VN == 0, "gelu_backward_bias: OC=%d must be a multiple of %d", OC, VN);
+    LLMK_REQUIRE(aligned16(d_in_out) && aligned16(inp), "gelu_backward_bias: pointers must be 16-byte aligned");
+    if (M == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    const int ny = bias_grad_ny(OC);
+    llmk::ProfScope prof("gelu_backward_bias", 0, 3.0 * M * OC * sizeof(floatX), st);
+    bias_grad_kernel<true><<<dim3(CEIL_DIV(OC, BG_COLV * VN), ny), 256, 0, st>>>(dbias_buffer, (floatX*)d_in_out, (const floatX*)inp, M, OC);
+    LAUNCH_CHECK();
+    bias_grad_reduce_kernel<<<CEIL_DIV(OC, BGR_COLS), BGR_COLS * BGR_GROUPS, 0, st>>>((floatX*)dbias, dbias_buffer, OC, ny);
+    LAUNCH_CHECK();
+}
+
 size_t llmk_matmul_backward_bias_scratch_floats(int OC) { return (size_t)bias_grad_ny(OC) * OC; }
 
 void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
@@ -564,7 +597,7 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         LLMK_REQUIRE(dbias_buffer != nullptr, "matmul_backward: dbias_buffer is required when dbias is given");
         const int ny = bias_grad_ny(OC);
         llmk::ProfScope prof("bias_grad", 0, (double)M * OC * sizeof(floatX), st);
-        bias_grad_kernel<<<dim3(CEIL_DIV(OC, BG_COLV * VN), ny), 256, 0, st>>>(dbias_buffer, (const floatX*)dout, M, OC);
+        bias_grad_kernel<false><<<dim3(CEIL_DIV(OC, BG_COLV * VN), ny), 256, 0, st>>>(dbias_buffer, (floatX*)dout, nullptr, M, OC);
         LAUNCH_CHECK();
         bias_grad_reduce_kernel<<<CEIL_DIV(OC, BGR_COLS), BGR_COLS * BGR_GROUPS, 0, st>>>((floatX*)dbias, dbias_buffer, OC, ny);
         LAUNCH_CHECK();
@@ -577,14 +610,24 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         g.M = M; g.N = C; g.K = OC; g.lda = OC; g.ldb = C; g.ldc = C;
         g.k_per_split = CEIL_DIV(OC, K_STEP) * K_STEP;
         const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(C, BIG_TILE) >= (size_t)num_cu;
+#if defined(LLMK_FP32)
         const bool fused = pre_gelu && gelu_fusion >= 2;
+#else
+        // bf16: gelu' in the epilogue costs the matrix cores more idle time than the extra elementwise pass takes
+        // (0.57 ms either way at (65536, 3072) on MI355X), so the GEMM stays plain and GELU backward runs after it.
+        const bool fused = false;
+        (void)gelu_fusion;
+#endif
         {
             llmk::ProfScope prof(fused ? "gemm_nn_dgelu" : "gemm_nn", 2.0 * M * (double)OC * C,
                                  ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
+#if defined(LLMK_FP32)
             if (fused) {
                 g.aux = (floatX*)pre_gelu;
                 launch_best<false, true, EPI_DGELU>(g, 1, big, st);
-            } else {
+            } else
+#endif
+            {
                 launch_best<false, true, EPI_STORE>(g, 1, big, st);
             }
         }

@@ -9,23 +9,24 @@
 //     classic "global -> registers -> ds_write" staging leaves the matrix cores idle while every
 //     wave writes LDS. Here operands go global -> LDS directly (global_load_lds_dwordx4): no
 //     staging registers, no ds_write instructions, and the LDS writes trickle in while MFMAs run.
-//   * K advances in blocks of 32 through a ring of five 32 KiB LDS slots (all 160 KiB of the CU); loads run
-//     four blocks (128 KiB per CU) ahead of the math, which is what it takes to cover HBM/L2 latency at
-//     this consumption rate. One s_barrier per block, without a memory fence (a fence would drain the ring).
+//   * K advances in stages of 64 through two 64 KiB LDS buffers: one is multiplied while the other fills. One
+//     stage ahead is enough to cover the latency (deeper rings of smaller blocks measured no faster), a stage of
+//     64 means every row of a K-contiguous operand is fetched as one full 128-byte line, and there is one
+//     s_barrier per 64 of K - without a memory fence, which would drain the loads in flight.
 //   * A direct-to-LDS load deposits each wave's 64 x 16 B linearly, so the anti-bank-conflict
 //     swizzle is applied on the global side: lane p of a row fetches chunk p ^ f(row), and the
-//     MFMA operand reads undo it. K-contiguous tiles: [row][32] with f = (row>>2)&3 (ds_read_b128
+//     MFMA operand reads undo it. K-contiguous tiles: [row][64] with f = (row>>1)&7 (ds_read_b128
 //     conflict-free). K-major tiles: [k][row] as in memory, f = 4*(k&3), read with the transposing
 //     ds_read_b64_tr_b16 so no software transpose is needed for dinp/dweight.
+//   * Operand reads are software-pipelined one 16-wide step ahead of the MFMAs, across the barrier.
+//   * The two waves that share a SIMD request their part of a stage at different points of the math.
 //   * The kernel is persistent (one workgroup per CU walks a list of tiles). When a tile's K loop
-//     ends, the first four K-blocks of the NEXT tile are requested into four ring slots while the
-//     epilogue stages its output through the fifth.
+//     ends, the first two stages of the NEXT tile are requested while the epilogue stages its output
+//     through a third LDS region.
 //   * The MFMA is issued with swapped operands (D^T = B.A^T): each lane then owns 4 consecutive
 //     output columns of one row, which it writes as 8 bytes into a per-wave LDS staging strip; the
 //     strip is read back row-contiguously so that global stores (and the loads of pre_gelu / the
 //     old dW for the fused epilogues) are full 128-byte lines.
-//   * Tile ids are dealt so that the 32 CUs of an XCD (which share an L2) work on an 8x4 patch of
-//     neighbouring tiles.
 #pragma once
 #include "common.hpp"
 #include "gelu.hpp"
@@ -57,11 +58,14 @@ struct GemmArgs {
 
 #if !defined(LLMK_FP32)
 
-constexpr int PBK = 32;                 // K per pipeline block
-constexpr int STAGES = 5;               // ring slots of one K block: two pairs of blocks and a spare for the epilogue
-constexpr int KGRAN = 2 * PBK;          // K (and the K range of a split) must be a multiple of this
+constexpr int PBK = 64;                 // K per stage
+constexpr int STAGES = 2;               // operand buffers: one being multiplied, one being filled
+constexpr int KGRAN = PBK;              // K (and the K range of a split) must be a multiple of this
 constexpr int LDS_TOTAL = 160 * 1024;
 constexpr int EPI_PITCH = 144;          // bytes per staged output row: 128 + 16
+
+// dynamic LDS of a launch: the operand buffers plus the epilogue's staging strips (16 rows per wave)
+constexpr int smem_bytes(int bm, int bn, int nw) { return STAGES * (bm + bn) * PBK * 2 + ((nw * 16 * EPI_PITCH + 1023) & ~1023); }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
@@ -94,6 +98,15 @@ __device__ __forceinline__ void st_cached(T* p, T v) {
     *p = v;
 }
 
+// transposing 8-byte LDS read at addr + OFF (see the kernel for why it is not the builtin)
+template <int OFF>
+__device__ __forceinline__ s16x4 ds_read_tr16(unsigned addr) {
+    static_assert(OFF >= 0 && OFF < 65536, "LDS instruction offsets are 16 bits");
+    s16x4 v;
+    asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFF));
+    return v;
+}
+
 // tile id -> tile coordinates; consecutive ids walk an 8-row group of tiles column by column
 __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int& tm, int& tn) {
     const int per_group = 8 * tiles_n;
@@ -116,18 +129,16 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int PASSES_OF_EPI = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
-    static_assert(STAGES * STAGE <= LDS_TOTAL, "LDS budget");
+    constexpr int STRIP = 16 * EPI_PITCH;                      // epilogue staging per wave: 16 rows x (128 B + 16 B pad)
+    constexpr int SPARE = (NW * STRIP + 1023) & ~1023;
+    static_assert(STAGES * STAGE + SPARE <= LDS_TOTAL, "LDS budget");
     static_assert(TN % 2 == 0, "epilogue strips are 64 columns wide");
     static_assert(A_CHUNKS % NW == 0, "each load slot of a wave must be all-A or all-B");
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
-    if (DBG & 64) {  // experiment: stagger the workgroups of an XCD over one tile period
-        const int phase = (blockIdx.x >> 3) & 7;
-        for (int i = 0; i < phase; i++) __builtin_amdgcn_s_sleep(100);
-    }
     if (DBG & 1) {   // ablation without loads: define the LDS contents (32: pseudo-random bits, else zeros)
-        for (int i = tid * 4; i < STAGES * STAGE; i += NT * 4) {
+        for (int i = tid * 4; i < STAGES * STAGE + SPARE; i += NT * 4) {
             unsigned v = (DBG & 32) ? ((squirrel_noise5((uint32_t)i, 17u) & 0x3fff3fffu) | 0x30003000u) : 0u;
             *reinterpret_cast<unsigned*>(lds + i) = v;
         }
@@ -137,7 +148,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     const int wm = wave / WGN, wn = wave % WGN;
     // The two waves that share a SIMD (w and w + NW/2) request their share of a K block at different points of
     // the block's math, so that a wave held up at the memory pipeline's entrance always has a partner issuing MFMAs.
-    const bool late = (DBG & 2048) ? false : wave >= NW / 2;
+    const bool late = wave >= NW / 2;
     const int idx = lane & 31, half = lane >> 5;
     const int tiles_m = CEIL_DIV(g.M, BM), tiles_n = CEIL_DIV(g.N, BN);
     const int num_tiles = tiles_m * tiles_n;
@@ -152,7 +163,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     const int G = gridDim.x;
     auto work_item = [&](int it, int& tm, int& tn, int& sp) -> bool {
         const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, per_x = G >> 3;
-        if (!(DBG & 65536) && g.splits == 1 && tiles_m >= 64) {
+        if (g.splits == 1 && tiles_m >= 64) {
             const int r0 = (tiles_m * xcd) >> 3, rows = ((tiles_m * (xcd + 1)) >> 3) - r0;
             const int q = it * per_x + local;
             if (q >= rows * tiles_n) return false;
@@ -169,81 +180,91 @@ gemm_pipelined_kernel(GemmArgs g) {
     };
 
     // --- per-thread load descriptors -----------------------------------------------------------
-    const floatX* gp[CPW];       // global address of this lane's 16 bytes for K block 0 of the current work item
+    // Each lane's 16 bytes of chunk i sit at (tile base of the operand) + voff[i]; the tile bases and the advance
+    // per stage are wave-uniform, so a load costs one 32-bit VGPR of address.
+    unsigned voff[CPW];          // byte offset of this lane's 16 bytes inside the operand's tile panel
     int lds_dst[CPW];            // wave-uniform byte offset of the chunk inside a stage
-    size_t kstep[CPW];           // elements to advance per K block
+    const char* tile_base[2];    // A and B panels of the current work item at its first K
+    size_t stage_step[2];        // bytes to advance per stage
     auto setup_loads = [&](int m0, int n0, int kbeg) {
+        tile_base[0] = reinterpret_cast<const char*>(A_T ? g.A + (size_t)kbeg * g.lda + m0 : g.A + (size_t)m0 * g.lda + kbeg);
+        tile_base[1] = reinterpret_cast<const char*>(B_T ? g.B + (size_t)kbeg * g.ldb + n0 : g.B + (size_t)n0 * g.ldb + kbeg);
+        stage_step[0] = (A_T ? (size_t)PBK * g.lda : (size_t)PBK) * sizeof(floatX);
+        stage_step[1] = (B_T ? (size_t)PBK * g.ldb : (size_t)PBK) * sizeof(floatX);
 #pragma unroll
         for (int i = 0; i < CPW; i++) {
             const int ci = wave + i * NW;
             const bool isA = i * NW < A_CHUNKS;                   // compile-time after unrolling
             const int cc = isA ? ci : ci - A_CHUNKS;
-            const floatX* base = isA ? g.A : g.B;
             const int ld = isA ? g.lda : g.ldb;
             const int r0 = isA ? m0 : n0, rmax = isA ? g.M : g.N;
             const bool trans = isA ? A_T : B_T;
-            constexpr int RA = BM, RB = BN;
-            const int R = isA ? RA : RB;
+            const int R = isA ? BM : BN;
             lds_dst[i] = (isA ? 0 : A_STAGE) + cc * 1024;
-            if (!trans && (DBG & 256)) {   // experiment (loads only): full 128-byte lines per row
+            if (!trans) {
                 const int row = cc * 8 + (lane >> 3), p = lane & 7;
-                gp[i] = base + (size_t)min(r0 + row, rmax - 1) * ld + kbeg + p * 8;
-                kstep[i] = (size_t)128 * ld;
-            } else if (!trans) {
-                const int row = cc * 16 + (lane >> 2), p = lane & 3;
-                const int c = p ^ ((row >> 2) & 3);
-                const int grow = min(r0 + row, rmax - 1);
-                gp[i] = base + (size_t)grow * ld + kbeg + c * 8;
-                kstep[i] = PBK;
+                const int c = p ^ ((row >> 1) & 7);
+                const int lrow = min(row, rmax - 1 - r0);         // rows past the edge re-read the last valid row
+                voff[i] = ((unsigned)lrow * (unsigned)ld + c * 8) * (unsigned)sizeof(floatX);
             } else {
                 const int byte = cc * 1024 + lane * 16;
                 const int krow = byte / (R * 2), p = (byte % (R * 2)) >> 4;
-                const int cn = (DBG & 16384) ? p : p ^ (4 * (krow & 3));
-                int col = r0 + cn * 8;
-                if (col >= rmax) col = r0;
-                gp[i] = base + (size_t)(kbeg + krow) * ld + col;
-                kstep[i] = (size_t)PBK * ld;
+                const int cn = p ^ (4 * (krow & 3));
+                const int lcol = (r0 + cn * 8 < rmax) ? cn * 8 : 0;
+                voff[i] = ((unsigned)krow * (unsigned)ld + lcol) * (unsigned)sizeof(floatX);
             }
         }
     };
-    // two consecutive K blocks at once, the two 64-byte halves of every 128-byte line requested back to back
-    auto issue2 = [&](int kb, int slot0, int slot1) {
-        char* stage0 = lds + slot0 * STAGE;
-        char* stage1 = lds + slot1 * STAGE;
+    auto issue = [&](int st, int buf) {
+        char* stage = lds + buf * STAGE;
         if (DBG & 1) return;
+        const char* pa = tile_base[0] + (size_t)st * stage_step[0];
+        const char* pb = tile_base[1] + (size_t)st * stage_step[1];
 #pragma unroll
-        for (int i = 0; i < CPW; i++) {
-            __builtin_amdgcn_global_load_lds(gp[i] + (size_t)kb * kstep[i], (lds_void_ptr)(stage0 + lds_dst[i]), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds(gp[i] + (size_t)(kb + 1) * kstep[i], (lds_void_ptr)(stage1 + lds_dst[i]), 16, 0, 0);
-        }
+        for (int i = 0; i < CPW; i++)
+            __builtin_amdgcn_global_load_lds((i * NW < A_CHUNKS ? pa : pb) + voff[i], (lds_void_ptr)(stage + lds_dst[i]), 16, 0, 0);
     };
 
     // --- MFMA operand reads ----------------------------------------------------------------------
-    auto frag_k = [&](const char* tile, int row0, int s) -> bf16x8 {        // K-contiguous tile [row][32]
-        const int row = row0 + idx, c = 2 * s + half;
-        return *reinterpret_cast<const bf16x8*>(tile + row * 64 + ((c ^ ((row >> 2) & 3)) << 4));
-    };
-    // The transposing reads are issued as inline asm on purpose: for the builtin, the compiler cannot tell that the
-    // read does not alias the in-flight direct-to-LDS loads and would wait for ALL of them (vmcnt(0)) first, which
-    // serialises loading and math. The price is that their completion has to be awaited by hand (lds_wait below).
-    auto frag_t = [&](const char* tile, int pitch, int row0, int s) -> bf16x8 {   // K-major tile [k][row], transposing read
+    // One LDS address per 32-row fragment and lane, for K step 0 of buffer 0; the other steps and the other buffer
+    // are reached by an XOR with the step (K-contiguous tiles: the swizzle is an XOR, so stepping the chunk index
+    // commutes with it) or an immediate offset (K-major tiles), so the loop keeps TM + TN address registers.
+    typedef __attribute__((address_space(3))) const char* lds_cptr;
+    const unsigned lds0 = (unsigned)(size_t)(lds_cptr)lds;                 // 1 KiB aligned
+    auto frag_base = [&](bool trans, int region, int rows, int row0) -> unsigned {
+        if (!trans) {
+            const int row = row0 + idx, f = (row >> 1) & 7;
+            return lds0 + region + row * 128 + ((f ^ half) << 4);
+        }
         const int s16 = lane & 15, grp = lane >> 4;
-        const int krow = 16 * s + 8 * (grp >> 1) + (s16 >> 2);             // (krow & 3) is the same for krow + 4
+        const int krow = 8 * (grp >> 1) + (s16 >> 2);                      // (krow & 3) is the same for krow + 4 and + 16 s
         const int col = row0 + (grp & 1) * 16 + 4 * (s16 & 3);
         const int cn = (col >> 3) ^ (4 * (krow & 3));
-        const char* p = tile + krow * pitch + cn * 16 + (col & 7) * 2;
-        const unsigned a0 = (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
-        const unsigned a1 = a0 + 4 * pitch;
-        s16x4 lo, hi;
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(a0));
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(hi) : "v"(a1));
+        return lds0 + region + krow * (rows * 2) + cn * 16 + (col & 7) * 2;
+    };
+    unsigned abase[TM], bbase[TN];
+#pragma unroll
+    for (int i = 0; i < TM; i++) abase[i] = frag_base(A_T, 0, BM, wm * WTM + i * 32);
+#pragma unroll
+    for (int j = 0; j < TN; j++) bbase[j] = frag_base(B_T, A_STAGE, BN, wn * WTN + j * 32);
+    // K-contiguous tile [row][64]: one 16-byte read
+    auto frag_k = [&](unsigned base, int s) -> bf16x8 {
+        return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)(base ^ (unsigned)(s << 5)));
+    };
+    // K-major tile [k][row]: two transposing 8-byte reads. They are issued as inline asm on purpose: for the builtin,
+    // the compiler cannot tell that the read does not alias the in-flight direct-to-LDS loads and would wait for ALL
+    // of them (vmcnt(0)) first, which serialises loading and math. The price is that their completion has to be
+    // awaited by hand (await_frags below).
+    auto frag_t = [&](unsigned base, auto off_lo, auto off_hi) -> bf16x8 {
         union { struct { s16x4 a, b; } s; bf16x8 v; } u;
-        u.s.a = lo; u.s.b = hi;
+        u.s.a = ds_read_tr16<decltype(off_lo)::value>(base);
+        u.s.b = ds_read_tr16<decltype(off_hi)::value>(base);
         return u.v;
     };
 
-    // fragments of one 16-wide K step
-    auto read_frags = [&](const char* sa, int s, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
+    // fragments of the 16-wide K step S of the buffer at byte offset bufoff
+    auto read_frags = [&](unsigned bufoff, auto sc, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
+        constexpr int S = decltype(sc)::value;
         if (DBG & 16) {
 #pragma unroll
             for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
@@ -251,17 +272,21 @@ gemm_pipelined_kernel(GemmArgs g) {
             for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
             return;
         }
-        const char* sb = sa + A_STAGE;
 #pragma unroll
-        for (int i = 0; i < TM; i++) fa[i] = A_T ? frag_t(sa, BM * 2, wm * WTM + i * 32, s) : frag_k(sa, wm * WTM + i * 32, s);
-        if (DBG & 512) {
-#pragma unroll
-            for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
-            return;
+        for (int i = 0; i < TM; i++) {
+            if constexpr (A_T) fa[i] = frag_t(abase[i] + bufoff, std::integral_constant<int, S * 16 * BM * 2>{}, std::integral_constant<int, (S * 16 + 4) * BM * 2>{});
+            else fa[i] = frag_k(abase[i] + bufoff, S);
         }
 #pragma unroll
-        for (int j = 0; j < TN; j++) fb[j] = B_T ? frag_t(sb, BN * 2, wn * WTN + j * 32, s) : frag_k(sb, wn * WTN + j * 32, s);
+        for (int j = 0; j < TN; j++) {
+            if constexpr (B_T) fb[j] = frag_t(bbase[j] + bufoff, std::integral_constant<int, S * 16 * BN * 2>{}, std::integral_constant<int, (S * 16 + 4) * BN * 2>{});
+            else fb[j] = frag_k(bbase[j] + bufoff, S);
+        }
     };
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+    using S2 = std::integral_constant<int, 2>;
+    using S3 = std::integral_constant<int, 3>;
     // Hand-issued (transposing) reads have to be awaited by hand. LDS operations return in order, so "at most
     // YOUNGER operations outstanding" means these operands have arrived when YOUNGER hand-issued reads were
     // requested after them (compiler-issued reads in between only make the wait longer). The operands are tied
@@ -290,51 +315,43 @@ gemm_pipelined_kernel(GemmArgs g) {
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
     };
     // Waiting for loads: vector-memory operations retire in issue order, so "at most N outstanding" means that
-    // everything but the N youngest has landed. The pairs of a tile are requested one at a time, so the only
-    // younger operations a wait ever has to allow are the second pair of the tile's prologue and the previous
+    // everything but the N youngest has landed. The stages of a tile are requested one at a time, so the only
+    // younger operations a wait ever has to allow are the second stage of the tile's prologue and the previous
     // tile's output stores (NS_EPI per wave when every lane stored, which holds for interior tiles).
     constexpr int NS_EPI = TM * PASSES_OF_EPI * 4 * (EPI == EPI_BIAS_GELU ? 2 : 1);
-    static_assert(2 * CPW + NS_EPI <= 63, "vmcnt is a 6-bit counter");
+    static_assert(CPW + NS_EPI <= 63, "vmcnt is a 6-bit counter");
 
-    int ring = 0;                       // ring slot that holds K block 0 of the current work item
     int it = 0;
     int tile_m, tile_n, split;
     if (!work_item(0, tile_m, tile_n, split)) return;
     int kbeg = split * g.k_per_split;
     int nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
     setup_loads(tile_m * BM, tile_n * BN, kbeg);
-    issue2(0, ring % STAGES, (ring + 1) % STAGES);
-    if (nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
+    issue(0, 0);
+    if (nkb > 1) issue(1, 1);
     bool st_young = false;              // the previous epilogue's stores are all issued and counted
 
     // Epilogues that read global memory (the pre-GELU activations, the old weight gradient) request it while the
     // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
     constexpr bool F32OUT = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
     constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
-    constexpr bool EPI_READS = (EPI == EPI_DGELU || EPI == EPI_ACCUM);
-    u32x4 pre_aux[EPI == EPI_DGELU ? TM : 1][2][2];
+    static_assert(EPI != EPI_DGELU, "GELU backward is not fused into this kernel");
+    constexpr bool EPI_READS = (EPI == EPI_ACCUM);
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
-    auto prefetch_epilogue = [&](int tm0, int tn0) {
-        if (!EPI_READS || (DBG & 4)) return;
+    auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
+        if (!EPI_READS || (DBG & 4) || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
 #pragma unroll
-        for (int i = 0; i < TM; i++)
+        for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
-            for (int pass = 0; pass < PASSES; pass++)
+            for (int hsel = 0; hsel < 2; hsel++)
 #pragma unroll
-                for (int hsel = 0; hsel < 2; hsel++)
-#pragma unroll
-                    for (int t = 0; t < 2; t++) {
-                        const int row = t * 8 + (lane >> 3), ch = lane & 7;
-                        const int m = wm0 + i * 32 + hsel * 16 + row;
-                        if (EPI == EPI_DGELU) {
-                            const int n = wn0 + pass * 64 + ch * 8;
-                            if (m < g.M && n < g.N) pre_aux[i][hsel][t] = *reinterpret_cast<const u32x4*>(g.aux + (size_t)m * g.ldc + n);
-                        } else {
-                            const int n = wn0 + pass * 32 + ch * 4;
-                            if (m < g.M && n < g.N) pre_old[i][pass][hsel][t] = *reinterpret_cast<const bf16x4*>(g.C + (size_t)m * g.ldc + n);
-                        }
-                    }
+                for (int t = 0; t < 2; t++) {
+                    const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                    const int m = wm0 + i * 32 + hsel * 16 + row;
+                    const int n = wn0 + pass * 32 + ch * 4;
+                    if (m < g.M && n < g.N) pre_old[i][pass][hsel][t] = *reinterpret_cast<const bf16x4*>(g.C + (size_t)m * g.ldc + n);
+                }
     };
 
     long long tc[8] = {0, 0, 0, 0, 0, 0, 0, 0};        // DBG & 128: cycle counts by phase (wave 0)
@@ -350,54 +367,53 @@ gemm_pipelined_kernel(GemmArgs g) {
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-        // ---- K loop over pairs of K blocks (one barrier per 64 of K), software-pipelined: the operands of the
-        // next 16-wide step (and the barrier that publishes the next pair) are requested while the matrix cores
-        // work on the current step. Pair p lives in ring slots 2p and 2p+1 (mod STAGES); while pair p is
-        // multiplied, pair p+1 is in flight and the fifth slot is spare (the epilogue's).
+        // ---- K loop over stages of 64, software-pipelined: the operands of the next 16-wide step (and the
+        // barrier that publishes the next stage) are requested while the matrix cores work on the current step.
+        // Stage s lives in buffer s & 1; while it is multiplied, stage s+1 is in flight.
         bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-        const int npairs = nkb >> 1;                              // the host guarantees an even number of K blocks
-        auto slot_of = [&](int kb) -> const char* { return lds + ((ring + kb) % STAGES) * STAGE; };
-        auto issue_pair = [&](int q) { issue2(2 * q, (ring + 2 * q) % STAGES, (ring + 2 * q + 1) % STAGES); };
+        const int nst = nkb;
+        auto buf_of = [&](int st) -> unsigned { return (unsigned)(st & 1) * STAGE; };
         long long ta = now();
-        if (npairs >= 2) { if (st_young) wait_vmcnt<2 * CPW + NS_EPI>(); else wait_vmcnt<2 * CPW>(); }
+        if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
         else wait_vmcnt<0>();
-        barrier_no_fence<DBG>();                                  // pair 0 landed for everyone
+        barrier_no_fence<DBG>();                                  // stage 0 landed for everyone
         long long tb = now();
         tc[0] += tb - ta;
         const long long t_loop = tb;
-        read_frags(slot_of(0), 0, fa0, fb0);
-        for (int p = 0; p < npairs - 1; p++) {
-            read_frags(slot_of(2 * p), 1, fa1, fb1);
+        read_frags(buf_of(0), S0{}, fa0, fb0);
+        for (int st = 0; st < nst - 1; st++) {
+            const unsigned cur = buf_of(st);
+            read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            if (late && p >= 1) issue_pair(p + 1);
-            read_frags(slot_of(2 * p + 1), 0, fa0, fb0);
+            if (late && st >= 1) issue(st + 1, (st + 1) & 1);
+            read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
-            read_frags(slot_of(2 * p + 1), 1, fa1, fb1);
+            read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading pair p
+            __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
             ta = now();
-            if (p == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // pair p+1 has landed (for this wave's share)
+            if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
             if (DBG & 128) { tb = now(); tc[6] += tb - ta; }
-            barrier_no_fence<DBG>();                              // ... and for everyone; the slots of pair p are free
+            barrier_no_fence<DBG>();                              // ... and for everyone; the buffer of stage st is free
             if (DBG & 128) { tb = now(); tc[2] += tb - ta; }
-            if (!late && p + 2 < npairs) issue_pair(p + 2);
-            read_frags(slot_of(2 * p + 2), 0, fa0, fb0);
+            if (!late && st + 2 < nst) issue(st + 2, st & 1);
+            read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
         }
         {
-            const int p = npairs - 1;
-            prefetch_epilogue(m0, n0);
-            read_frags(slot_of(2 * p), 1, fa1, fb1);
+            const unsigned cur = buf_of(nst - 1);
+            prefetch_epilogue(m0, n0, 0);
+            read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            read_frags(slot_of(2 * p + 1), 0, fa0, fb0);
+            read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
-            read_frags(slot_of(2 * p + 1), 1, fa1, fb1);
+            read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
             await_frags(fa1, fb1, NoneYounger{});
@@ -406,9 +422,9 @@ gemm_pipelined_kernel(GemmArgs g) {
         if (DBG & 128) { ta = now(); tc[3] += ta - t_loop; }
 
         // ---- request the next work item's first K blocks, then run the epilogue under them --------
-        barrier_no_fence<DBG>();                                       // every wave is done reading the ring
-        const int ring_free = (ring + nkb) % STAGES;              // slot the epilogue may use
+        barrier_no_fence<DBG>();                                  // every wave is done reading both buffers
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
+        prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
         it++;
         const bool have_next = work_item(it, tile_m, tile_n, split);
         int next_nkb = 0;
@@ -416,18 +432,14 @@ gemm_pipelined_kernel(GemmArgs g) {
             kbeg = split * g.k_per_split;
             next_nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
             setup_loads(tile_m * BM, tile_n * BN, kbeg);
-            ring = (ring_free + 1) % STAGES;
-            issue2(0, ring % STAGES, (ring + 1) % STAGES);
-            if (!(DBG & 8192) && next_nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
+            issue(0, 0);
+            if (next_nkb > 1) issue(1, 1);
         }
 
         // ---- epilogue ---------------------------------------------------------------------------------
-        // wave-private staging strip inside the free ring slot: 16 rows x (128 B + 16 B pad)
+        // wave-private staging strip behind the operand buffers: 16 rows x (128 B + 16 B pad)
         {
-            constexpr int STRIP_ROWS = 16;
-            constexpr int STRIP = STRIP_ROWS * EPI_PITCH;
-            static_assert(NW * STRIP <= STAGE, "all strips must fit in one ring slot");
-            char* strip = lds + ring_free * STAGE + wave * STRIP;
+            char* strip = lds + STAGES * STAGE + wave * STRIP;
             const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
             constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
 #pragma unroll
@@ -497,17 +509,12 @@ gemm_pipelined_kernel(GemmArgs g) {
                                 const int n = wn0 + pass * 64 + ch * 8;
                                 if (m < g.M && n < g.N && !(DBG & 4)) {
                                     const size_t o = (size_t)m * g.ldc + n;
-                                    union { u32x4 u; bf16x8 h; } x, y, z;
+                                    union { u32x4 u; bf16x8 h; } x, y;
                                     x.u = raw;
                                     if (EPI == EPI_BIAS_GELU) {
                                         st_out<DBG>(reinterpret_cast<u32x4*>(g.aux + o), x.u);
 #pragma unroll
                                         for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
-                                    } else if (EPI == EPI_DGELU) {
-                                        z.u = pre_aux[EPI == EPI_DGELU ? i : 0][hsel][t];
-#pragma unroll
-                                        for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)z.h[e]) * (float)x.h[e]);
                                         st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                     } else {
                                         st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), x.u);
@@ -519,12 +526,12 @@ gemm_pipelined_kernel(GemmArgs g) {
                         __builtin_amdgcn_wave_barrier();
                     }
                 }
+                prefetch_epilogue(cur_m0, cur_n0, i + 2);
             }
         }
-        if ((DBG & 8192) && have_next && next_nkb > 2) issue2(2, (ring + 2) % STAGES, (ring + 3) % STAGES);
         if (DBG & 128) { tb = now(); tc[4] += tb - ta; }
         if (!have_next) break;
-        st_young = (DBG & 8192) ? false : cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
+        st_young = cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
         nkb = next_nkb;
     }
     if ((DBG & 128) && lane == 0) {

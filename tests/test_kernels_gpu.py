@@ -169,6 +169,40 @@ def test_gelu(precision):
     close(G.host(d_g), rd, **tol(precision, 1e-5, bf16_atol=1e-2))
 
 
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("N,OC", [(37, 64), (300, 3072), (2048, 264)])
+def test_gelu_backward_bias_equals_the_two_separate_steps(precision, N, OC):
+    """d *= gelu'(x) and dbias += colsum(d) in one pass: the GELU part against the oracle, the bias part against
+    what llmk_matmul_backward's bias step gives on the stored result (same summation order: bit-identical in bf16)."""
+    L = G.lib(precision)
+    x = G.rounded(rnd((N, OC), 0, 2.0), precision)
+    g = G.rounded(rnd((N, OC), 1), precision)
+    b0 = G.rounded(rnd(OC, 2), precision)
+    rd = np.zeros((N, OC), np.float32); ol.cref().cref_gelu_backward(rd, x, g, N * OC)
+    nscr = L.llmk_matmul_backward_bias_scratch_floats(OC)
+    d_x, d_g, d_b = G.dev(x, precision), G.dev(g, precision), G.dev(b0, precision)
+    d_s = G.dev(np.zeros(nscr, np.float32), "fp32")
+    L.llmk_gelu_backward_bias(G.ptr(d_g), G.ptr(d_x), G.ptr(d_b), G.ptr(d_s), 1, N, OC, None)
+    got_d, got_b = G.host(d_g), G.host(d_b)
+    close(got_d, rd, **tol(precision, 1e-5, bf16_atol=1e-2))
+    # the two-step path: same elementwise kernel semantics, then the library's own bias reduction on that result
+    d_g2, d_b2 = G.dev(g, precision), G.dev(b0, precision)
+    L.llmk_gelu_backward_inplace(G.ptr(d_g2), G.ptr(d_x), N * OC, None)
+    assert np.array_equal(G.host(d_g2), got_d)
+    C_in = 8
+    d_inp = G.dev(np.zeros((N, C_in), np.float32), precision); d_w = G.dev(np.zeros((OC, C_in), np.float32), precision)
+    d_dinp = G.dev(np.zeros((N, C_in), np.float32), precision); d_dw = G.dev(np.zeros((OC, C_in), np.float32), precision)
+    L.llmk_matmul_backward(G.ptr(d_dinp), G.ptr(d_dw), G.ptr(d_b2), G.ptr(d_g2), G.ptr(d_inp), G.ptr(d_w), G.ptr(d_s),
+                           1, N, C_in, OC, None, None, 1)
+    if precision == "bf16":
+        assert np.array_equal(G.host(d_b2), got_b)
+    else:                                   # fp32 storage: no rounding between product and sum, the compiler may fuse them
+        close(got_b, G.host(d_b2), rtol=1e-5, atol=1e-5)
+    # and against a float64 column sum
+    ref_b = b0.astype(np.float64) + got_d.astype(np.float64).sum(0)
+    close(got_b, ref_b.astype(np.float32), **tol(precision, 1e-4, bf16_rel=1e-2, bf16_atol=2e-2))
+
+
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("N,V,P", [(5, 100, 128), (64, 50257, 50304), (3, 8003, 8064), (2, 130000, 130048)])
