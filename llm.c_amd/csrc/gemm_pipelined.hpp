@@ -62,10 +62,9 @@ constexpr int PBK = 64;                 // K per stage
 constexpr int STAGES = 2;               // operand buffers: one being multiplied, one being filled
 constexpr int KGRAN = PBK;              // K (and the K range of a split) must be a multiple of this
 constexpr int LDS_TOTAL = 160 * 1024;
-constexpr int EPI_PITCH = 144;          // bytes per staged output row: 128 + 16
 
-// dynamic LDS of a launch: the operand buffers plus the epilogue's staging strips (16 rows per wave)
-constexpr int smem_bytes(int bm, int bn, int nw) { return STAGES * (bm + bn) * PBK * 2 + ((nw * 16 * EPI_PITCH + 1023) & ~1023); }
+// dynamic LDS of a launch: the operand buffers plus the epilogue's staging strips (32 rows of 128 B per wave)
+constexpr int smem_bytes(int bm, int bn, int nw) { return STAGES * (bm + bn) * PBK * 2 + nw * 32 * 128; }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
 
@@ -129,7 +128,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int PASSES_OF_EPI = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
-    constexpr int STRIP = 16 * EPI_PITCH;                      // epilogue staging per wave: 16 rows x (128 B + 16 B pad)
+    constexpr int STRIP = 32 * 128;                            // epilogue staging per wave: 32 rows x 128 B
     constexpr int SPARE = (NW * STRIP + 1023) & ~1023;
     static_assert(STAGES * STAGE + SPARE <= LDS_TOTAL, "LDS budget");
     static_assert(TN % 2 == 0, "epilogue strips are 64 columns wide");
@@ -186,11 +185,14 @@ gemm_pipelined_kernel(GemmArgs g) {
     int lds_dst[CPW];            // wave-uniform byte offset of the chunk inside a stage
     const char* tile_base[2];    // A and B panels of the current work item at its first K
     size_t stage_step[2];        // bytes to advance per stage
-    auto setup_loads = [&](int m0, int n0, int kbeg) {
+    auto setup_bases = [&](int m0, int n0, int kbeg) {
         tile_base[0] = reinterpret_cast<const char*>(A_T ? g.A + (size_t)kbeg * g.lda + m0 : g.A + (size_t)m0 * g.lda + kbeg);
         tile_base[1] = reinterpret_cast<const char*>(B_T ? g.B + (size_t)kbeg * g.ldb + n0 : g.B + (size_t)n0 * g.ldb + kbeg);
         stage_step[0] = (A_T ? (size_t)PBK * g.lda : (size_t)PBK) * sizeof(floatX);
         stage_step[1] = (B_T ? (size_t)PBK * g.ldb : (size_t)PBK) * sizeof(floatX);
+    };
+    // the lane offsets depend on the tile only through the clamping at the matrix edges: interior tiles share them
+    auto setup_voff = [&](int m0, int n0) {
 #pragma unroll
         for (int i = 0; i < CPW; i++) {
             const int ci = wave + i * NW;
@@ -326,7 +328,10 @@ gemm_pipelined_kernel(GemmArgs g) {
     if (!work_item(0, tile_m, tile_n, split)) return;
     int kbeg = split * g.k_per_split;
     int nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
-    setup_loads(tile_m * BM, tile_n * BN, kbeg);
+    auto is_edge = [&](int tm, int tn) -> bool { return tm * BM + BM > g.M || tn * BN + BN > g.N; };
+    bool voff_edge = is_edge(tile_m, tile_n);
+    setup_bases(tile_m * BM, tile_n * BN, kbeg);
+    setup_voff(tile_m * BM, tile_n * BN);
     issue(0, 0);
     if (nkb > 1) issue(1, 1);
     bool st_young = false;              // the previous epilogue's stores are all issued and counted
@@ -372,6 +377,9 @@ gemm_pipelined_kernel(GemmArgs g) {
         // Stage s lives in buffer s & 1; while it is multiplied, stage s+1 is in flight.
         bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
         const int nst = nkb;
+        // the next work item's coordinates are worked out here (integer divisions), under the K loop's MFMAs
+        int next_m, next_n, next_split;
+        const bool have_next = work_item(it + 1, next_m, next_n, next_split);
         auto buf_of = [&](int st) -> unsigned { return (unsigned)(st & 1) * STAGE; };
         long long ta = now();
         if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
@@ -423,108 +431,111 @@ gemm_pipelined_kernel(GemmArgs g) {
 
         // ---- request the next work item's first K blocks, then run the epilogue under them --------
         barrier_no_fence<DBG>();                                  // every wave is done reading both buffers
+        if (DBG & 128) { tb = now(); tc[1] += tb - ta; }
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
         prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
         it++;
-        const bool have_next = work_item(it, tile_m, tile_n, split);
         int next_nkb = 0;
         if (have_next) {
+            tile_m = next_m; tile_n = next_n; split = next_split;
             kbeg = split * g.k_per_split;
             next_nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
-            setup_loads(tile_m * BM, tile_n * BN, kbeg);
+            setup_bases(tile_m * BM, tile_n * BN, kbeg);
+            const bool edge = is_edge(tile_m, tile_n);
+            if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
+            voff_edge = edge;
             issue(0, 0);
             if (next_nkb > 1) issue(1, 1);
         }
+        if (DBG & 128) { long long tcur = now(); tc[7] += tcur - tb; }
 
         // ---- epilogue ---------------------------------------------------------------------------------
-        // wave-private staging strip behind the operand buffers: 16 rows x (128 B + 16 B pad)
+        // Wave-private staging strip behind the operand buffers: 32 rows x 128 B, the 16-byte chunk c of row r stored
+        // at chunk c ^ ((r >> 1) & 7). One 32-row block of the wave's tile goes through it at a time: every lane
+        // writes the 4-column pieces it owns, then the wave reads the rows back 8 lanes to a row and stores
+        // full 128-byte lines.
         {
             char* strip = lds + STAGES * STAGE + wave * STRIP;
             const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
             constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
+            const int wswz = (idx >> 1) & 7;
 #pragma unroll
             for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++) {
+                    // phase 1: lane (row = idx, half) owns columns 8q + 4*half + 0..3 of each 32-column block
 #pragma unroll
-                    for (int hsel = 0; hsel < 2; hsel++) {        // rows 0..15 / 16..31 of the 32-row block
-                        // phase 1: lane (m = idx, half) owns n = 8q + 4*half + 0..3 of each 32-column block
-                        if ((idx >> 4) == hsel) {
+                    for (int j = pass * JP; j < (pass + 1) * JP; j++) {
 #pragma unroll
-                            for (int j = pass * JP; j < (pass + 1) * JP; j++) {
+                        for (int q = 0; q < 4; q++) {
+                            const int nl = j * 32 + 8 * q + 4 * half;                 // column inside the wave tile
+                            float v[4];
 #pragma unroll
-                                for (int q = 0; q < 4; q++) {
-                                    const int nl = j * 32 + 8 * q + 4 * half;                 // column inside the wave tile
-                                    const int sl = (j - pass * JP) * 32 + 8 * q + 4 * half;   // column inside the strip
-                                    float v[4];
+                            for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
+                            if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+                                if (g.bias) {
+                                    const int n = wn0 + nl;
+                                    if (n < g.N) {
+                                        bf16x4 b4 = *reinterpret_cast<const bf16x4*>(g.bias + n);
 #pragma unroll
-                                    for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
-                                    if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
-                                        if (g.bias) {
-                                            const int n = wn0 + nl;
-                                            if (n < g.N) {
-                                                bf16x4 b4 = *reinterpret_cast<const bf16x4*>(g.bias + n);
-#pragma unroll
-                                                for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
-                                            }
-                                        }
-                                    }
-                                    char* dst = strip + (idx & 15) * EPI_PITCH;
-                                    if (F32OUT) {
-                                        f32x4 o = {v[0], v[1], v[2], v[3]};
-                                        *reinterpret_cast<f32x4*>(dst + (8 * q + 4 * half) * 4) = o;
-                                    } else {
-                                        bf16x4 o;
-#pragma unroll
-                                        for (int e = 0; e < 4; e++) o[e] = (__bf16)v[e];
-                                        *reinterpret_cast<bf16x4*>(dst + sl * 2) = o;
+                                        for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
                                     }
                                 }
                             }
-                        }
-                        __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): the strip is written
-                        __builtin_amdgcn_wave_barrier();
-                        // phase 2: 16 rows x 128 B, 8 lanes per row
+                            char* dst = strip + idx * 128;
+                            if (F32OUT) {                         // 16 bytes: chunk 2q + half
+                                f32x4 o = {v[0], v[1], v[2], v[3]};
+                                *reinterpret_cast<f32x4*>(dst + (((2 * q + half) ^ wswz) << 4)) = o;
+                            } else {                              // 8 bytes: half of chunk 4(j - pass*JP) + q
+                                bf16x4 o;
 #pragma unroll
-                        for (int t = 0; t < 2; t++) {
-                            const int row = t * 8 + (lane >> 3), ch = lane & 7;
-                            const int m = wm0 + i * 32 + hsel * 16 + row;
-                            u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * EPI_PITCH + ch * 16);
-                            if (F32OUT) {
-                                const int n = wn0 + pass * 32 + ch * 4;
-                                if (m < g.M && n < g.N && !(DBG & 4)) {
-                                    if (EPI == EPI_PARTIAL) {
-                                        st_cached(reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n), raw);
-                                    } else {
-                                        union { u32x4 u; f32x4 f; } x;
-                                        x.u = raw;
-                                        floatX* cp = g.C + (size_t)m * g.ldc + n;
-                                        bf16x4 old = pre_old[EPI == EPI_ACCUM ? i : 0][EPI == EPI_ACCUM ? pass : 0][hsel][t], o4;
-#pragma unroll
-                                        for (int e = 0; e < 4; e++) o4[e] = (__bf16)((float)old[e] + x.f[e]);
-                                        st_cached(reinterpret_cast<bf16x4*>(cp), o4);
-                                    }
-                                }
-                            } else {
-                                const int n = wn0 + pass * 64 + ch * 8;
-                                if (m < g.M && n < g.N && !(DBG & 4)) {
-                                    const size_t o = (size_t)m * g.ldc + n;
-                                    union { u32x4 u; bf16x8 h; } x, y;
-                                    x.u = raw;
-                                    if (EPI == EPI_BIAS_GELU) {
-                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.aux + o), x.u);
-#pragma unroll
-                                        for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
-                                    } else {
-                                        st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), x.u);
-                                    }
-                                }
+                                for (int e = 0; e < 4; e++) o[e] = (__bf16)v[e];
+                                *reinterpret_cast<bf16x4*>(dst + ((((j - pass * JP) * 4 + q) ^ wswz) << 4) + half * 8) = o;
                             }
                         }
-                        __builtin_amdgcn_s_waitcnt(0xC07F);          // strip reads done before it is overwritten
-                        __builtin_amdgcn_wave_barrier();
                     }
+                    __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): the strip is written
+                    __builtin_amdgcn_wave_barrier();
+                    // phase 2: 32 rows x 128 B, 8 lanes per row
+#pragma unroll
+                    for (int t = 0; t < 4; t++) {
+                        const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                        const int m = wm0 + i * 32 + row;
+                        u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4));
+                        if (F32OUT) {
+                            const int n = wn0 + pass * 32 + ch * 4;
+                            if (m < g.M && n < g.N && !(DBG & 4)) {
+                                if (EPI == EPI_PARTIAL) {
+                                    st_cached(reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n), raw);
+                                } else {
+                                    union { u32x4 u; f32x4 f; } x;
+                                    x.u = raw;
+                                    floatX* cp = g.C + (size_t)m * g.ldc + n;
+                                    bf16x4 old = pre_old[EPI == EPI_ACCUM ? i : 0][EPI == EPI_ACCUM ? pass : 0][t >> 1][t & 1], o4;
+#pragma unroll
+                                    for (int e = 0; e < 4; e++) o4[e] = (__bf16)((float)old[e] + x.f[e]);
+                                    st_cached(reinterpret_cast<bf16x4*>(cp), o4);
+                                }
+                            }
+                        } else {
+                            const int n = wn0 + pass * 64 + ch * 8;
+                            if (m < g.M && n < g.N && !(DBG & 4)) {
+                                const size_t o = (size_t)m * g.ldc + n;
+                                union { u32x4 u; bf16x8 h; } x, y;
+                                x.u = raw;
+                                if (EPI == EPI_BIAS_GELU) {
+                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.aux + o), x.u);
+#pragma unroll
+                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
+                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                } else {
+                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), x.u);
+                                }
+                            }
+                        }
+                    }
+                    __builtin_amdgcn_s_waitcnt(0xC07F);          // strip reads done before it is overwritten
+                    __builtin_amdgcn_wave_barrier();
                 }
                 prefetch_epilogue(cur_m0, cur_n0, i + 2);
             }
