@@ -32,6 +32,7 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 constexpr int HS = 64;
+constexpr int FA_FWD_WAVES = 4;       // waves (of 32 queries) per forward workgroup
 constexpr int KP = 144;               // LDS pitch (bytes) of a [row][64 x bf16] tile: 128 + 16, conflict-free for
                                       // both ds_read_b128 down a column of rows and the transposing 8-byte reads
 constexpr int TILE_BYTES = 64 * KP;   // 64 rows
@@ -93,19 +94,42 @@ __device__ __forceinline__ void store4(floatX* p, float a, float b, float c, flo
     *reinterpret_cast<bf16x4*>(p) = o;
 }
 
+// Which (tile along T, batch*head) a workgroup works on. The grid is (tiles, B*NH) with x fastest, and workgroups
+// are dealt round-robin over the 8 XCDs, each with its own L2: taken literally, the tiles of one head would land
+// on 8 different XCDs and each would pull that head's K and V through its own L2. Instead XCD x takes the heads
+// x, x+8, ... and walks all tiles of a head with consecutive workgroups, so a head's K/V cross HBM once.
+__device__ __forceinline__ void fa_block_coords(int& tile, int& bh) {
+    const int nt = gridDim.x, nbh = gridDim.y;
+    tile = blockIdx.x; bh = blockIdx.y;
+    if ((nbh & 7) == 0) {
+        const int lin = blockIdx.y * nt + blockIdx.x;
+        const int xcd = lin & 7, slot = lin >> 3;
+        bh = (slot / nt) * 8 + xcd;
+        tile = slot % nt;
+    }
+}
+
 // ---- forward ----------------------------------------------------------------------------------
-// grid (ceil(T/128), B*NH), 256 threads: wave w owns queries [128*qt + 32w, +32)
-__global__ void __launch_bounds__(256)
+// grid (ceil(T/128), B*NH), 256 threads: wave w owns queries [128*qt + 32w, +32) and walks the key tiles up to
+// its diagonal, 32 keys at a time. The loop is bound by the vector ALU (one exp2 per score costs as much as the
+// two MFMAs that score takes part in), so everything else per score is kept to a minimum: the first MFMA of a
+// block starts from a constant zero instead of a cleared accumulator, maxima are taken three at a time, and the
+// K/V staging loads use a wave-uniform base with per-thread offsets that never change.
+template <int NWAVES = 8, int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no K/V streaming, 4: no barrier)
+__global__ void __launch_bounds__(NWAVES * 64)
 fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
     __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char sV[2][TILE_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
-    const int qt = gridDim.x - 1 - blockIdx.x;          // longest rows first
-    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    int tile_x, bh;
+    fa_block_coords(tile_x, bh);
+    const int qt = gridDim.x - 1 - tile_x;              // longest rows first
+    const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
     const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
-    const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+    constexpr int GQ = 32 * NWAVES, NT = 64 * NWAVES, NLD = 512 / NT;   // queries per workgroup, threads, 16-byte loads per thread and tile
+    const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
     const float c = 0.125f * LOG2E;                       // 1/sqrt(64) folded into the exp2 argument
 
     bf16x8 qf[4];
@@ -121,91 +145,115 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
     for (int d = 0; d < 2; d++)
 #pragma unroll
         for (int r = 0; r < 16; r++) o[d][r] = 0.f;
-    float m = -INFINITY, l = 0.f;
+    float m = -INFINITY;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // The softmax denominator is accumulated by the matrix cores, which have cycles to spare here: a ones operand
+    // in place of V makes every row of this accumulator the sum over keys of the (bf16-rounded) probabilities of
+    // the lane's query - the same rounded values that multiply V.
+    f32x16 lacc = zero;
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ones[e] = (__bf16)1.0f;
 
-    const int last_q = min(qt * 128 + 127, T - 1);
+    const int last_q = min(qt * GQ + GQ - 1, T - 1);
     const int n_kt = last_q / 64 + 1;
-    TileRegs rk, rv;
-    tile_load(rk, base + C, C3, 0, T, tid);
-    tile_load(rv, base + 2 * C, C3, 0, T, tid);
-    tile_store(sK[0], rk, tid);
-    tile_store(sV[0], rv, tid);
+    // staging: thread (row = tid/8, chunk = tid%8) copies NLD rows, NT/8 apart, of the K and of the V tile
+    const int srow = tid >> 3, schunk = tid & 7;
+    const unsigned g_off = (unsigned)((size_t)srow * C3 + schunk * 8) * (unsigned)sizeof(floatX);
+    const unsigned g_step = (unsigned)((NT / 8) * C3 * sizeof(floatX));
+    const int l_off = srow * KP + schunk * 16;
+    const char* kbase = reinterpret_cast<const char*>(base + C);
+    const char* vbase = reinterpret_cast<const char*>(base + 2 * C);
+    const size_t tile_step = 64 * C3 * sizeof(floatX);
+    u32x4 rk[NLD], rv[NLD];
+    auto stage_load = [&](int j) {
+        const char* pk = kbase + (size_t)j * tile_step;
+        const char* pv = vbase + (size_t)j * tile_step;
+        const u32x4 z = {0, 0, 0, 0};
+        if (64 * j + 64 <= T) {                          // whole tile inside the sequence (wave-uniform)
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                rk[i] = *reinterpret_cast<const u32x4*>(pk + g_off + i * g_step);
+                rv[i] = *reinterpret_cast<const u32x4*>(pv + g_off + i * g_step);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NLD; i++) {
+                const bool in = 64 * j + srow + i * (NT / 8) < T;
+                rk[i] = in ? *reinterpret_cast<const u32x4*>(pk + g_off + i * g_step) : z;
+                rv[i] = in ? *reinterpret_cast<const u32x4*>(pv + g_off + i * g_step) : z;
+            }
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < NLD; i++) {
+            *reinterpret_cast<u32x4*>(sK[buf] + l_off + i * (NT / 8) * KP) = rk[i];
+            *reinterpret_cast<u32x4*>(sV[buf] + l_off + i * (NT / 8) * KP) = rv[i];
+        }
+    };
+    stage_load(0);
+    stage_store(0);
     __syncthreads();
 
     for (int j = 0; j < n_kt; j++) {
-        const char* tk = sK[j & 1];
-        const char* tv = sV[j & 1];
-        const bool more = j + 1 < n_kt;
-        if (more) {
-            tile_load(rk, base + C, C3, 64 * (j + 1), T, tid);
-            tile_load(rv, base + 2 * C, C3, 64 * (j + 1), T, tid);
-        }
+        const char* tk = sK[(ABL & 2) ? 0 : (j & 1)];
+        const char* tv = sV[(ABL & 2) ? 0 : (j & 1)];
+        const bool more = j + 1 < n_kt && !(ABL & 2);
+        if (more) stage_load(j + 1);
         if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
+            // S^T for both 32-key blocks, the two accumulation chains interleaved
             f32x16 sacc[2];
-            const bool kb1 = 64 * j + 32 <= qw0 + 31;     // second 32-key block not entirely masked
+            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 0, 0, lane), qf[0], zero, 0, 0, 0);
+            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32, 0, lane), qf[0], zero, 0, 0, 0);
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-                for (int r = 0; r < 16; r++) sacc[kb][r] = 0.f;
-                if (kb == 0 || kb1) {
-#pragma unroll
-                    for (int s = 0; s < 4; s++)
-                        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32 * kb, s, lane), qf[s], sacc[kb], 0, 0, 0);
-                }
+            for (int s = 1; s < 4; s++) {
+                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 0, s, lane), qf[s], sacc[0], 0, 0, 0);
+                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32, s, lane), qf[s], sacc[1], 0, 0, 0);
             }
             if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
+                asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int key = 64 * j + 32 * kb + acc_row(r, lane);
-                        if (key > my_q) sacc[kb][r] = -INFINITY;
-                    }
+                    for (int r = 0; r < 16; r++)
+                        if (64 * j + 32 * kb + acc_row(r, lane) > my_q) sacc[kb][r] = -INFINITY;
             }
-            float mx = -INFINITY;
+            float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) mx = fmaxf(mx, sacc[kb][r]);
+            for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
             const float m_new = fmaxf(m, mx * c);
             if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // some row's running max moved: rescale (rare after the first tiles)
+                asm volatile("" ::: "memory");
                 const float alpha = fast_exp2(m - m_new);
                 m = m_new;
-                l *= alpha;
+#pragma unroll
+                for (int r = 0; r < 16; r++) lacc[r] *= alpha;
 #pragma unroll
                 for (int d = 0; d < 2; d++)
 #pragma unroll
                     for (int r = 0; r < 16; r++) o[d][r] *= alpha;
             }
-            float rs = 0.f;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    float p = fast_exp2(fmaf(sacc[kb][r], c, -m));
-                    sacc[kb][r] = p;
-                    rs += p;
-                }
-            l += rs;
+                for (int r = 0; r < 16; r++)
+                    sacc[kb][r] = (ABL & 1) ? fmaf(sacc[kb][r], c, -m) : fast_exp2(fmaf(sacc[kb][r], c, -m));
 #pragma unroll
             for (int s2 = 0; s2 < 4; s2++) {
-                if (s2 < 2 || kb1) {
-                    bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
+                const bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
+                lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, lacc, 0, 0, 0);       // every row: sum over keys of P
 #pragma unroll
-                    for (int d = 0; d < 2; d++)
-                        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tv, 16 * s2, 32 * d, lane), pf, o[d], 0, 0, 0);
-                }
+                for (int d = 0; d < 2; d++)
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tv, 16 * s2, 32 * d, lane), pf, o[d], 0, 0, 0);
             }
         }
-        if (more) {
-            tile_store(sK[(j + 1) & 1], rk, tid);
-            tile_store(sV[(j + 1) & 1], rv, tid);
-        }
-        __syncthreads();
+        if (more) stage_store((j + 1) & 1);
+        if (!(ABL & 4)) __syncthreads();
     }
 
-    l += __shfl_xor(l, 32, WAVE);
+    const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
     if (my_q < T) {
         const float inv = 1.0f / l;
         floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
@@ -253,8 +301,9 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
     __shared__ __attribute__((aligned(16))) float sL[2][64];
     __shared__ __attribute__((aligned(16))) float sD[2][64];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
-    const int kt = blockIdx.x;
-    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    int kt, bh;
+    fa_block_coords(kt, bh);
+    const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
     const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
@@ -385,8 +434,10 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
     __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
     __shared__ __attribute__((aligned(16))) char sV[2][TILE_BYTES];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
-    const int qt = gridDim.x - 1 - blockIdx.x;
-    const int b = blockIdx.y / NH, h = blockIdx.y % NH;
+    int tile_x, bh;
+    fa_block_coords(tile_x, bh);
+    const int qt = gridDim.x - 1 - tile_x;
+    const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
     const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
@@ -586,7 +637,7 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 #if !defined(LLMK_FP32)
     LLMK_REQUIRE(hs == HS, "attention_forward: head size %d unsupported (bf16 build handles 64)", hs);
     LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
-    fa_forward_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+    fa_forward_kernel<FA_FWD_WAVES><<<dim3(CEIL_DIV(T, 32 * FA_FWD_WAVES), B * NH), 64 * FA_FWD_WAVES, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
 #else
     LLMK_REQUIRE(hs <= 64, "attention_forward: head size %d unsupported (fp32 build handles <= 64)", hs);
     const size_t rows = (size_t)B * NH * T;
