@@ -72,20 +72,26 @@ __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + 
 
 // cooperative 64x64 bf16 tile copy global -> registers (2 x 16 B per thread, 256 threads)
 struct TileRegs { u32x4 v[2]; };
-__device__ __forceinline__ void tile_load(TileRegs& t, const floatX* base, size_t row_stride, int row0, int nrows, int tid) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int q = tid + i * 256, row = q >> 3, c = q & 7;
-        u32x4 z = {0, 0, 0, 0};
-        t.v[i] = (row0 + row < nrows) ? *reinterpret_cast<const u32x4*>(base + (size_t)(row0 + row) * row_stride + c * 8) : z;
+// `tile` points at the first row of the tile (wave-uniform); thread (row = tid/8, chunk = tid%8) copies rows row and
+// row+32. The per-thread part of the address never changes from tile to tile, so it is 32-bit and loop-invariant.
+__device__ __forceinline__ void tile_load(TileRegs& t, const floatX* tile, size_t row_stride, int rows_left, int tid) {
+    const char* p = reinterpret_cast<const char*>(tile);
+    const int row = tid >> 3;
+    const unsigned off0 = (unsigned)((size_t)row * row_stride + (tid & 7) * 8) * (unsigned)sizeof(floatX);
+    const unsigned off1 = off0 + (unsigned)(32 * row_stride * sizeof(floatX));
+    if (rows_left >= 64) {                                // whole tile inside the sequence (wave-uniform)
+        t.v[0] = *reinterpret_cast<const u32x4*>(p + off0);
+        t.v[1] = *reinterpret_cast<const u32x4*>(p + off1);
+    } else {
+        const u32x4 z = {0, 0, 0, 0};
+        t.v[0] = row < rows_left ? *reinterpret_cast<const u32x4*>(p + off0) : z;
+        t.v[1] = row + 32 < rows_left ? *reinterpret_cast<const u32x4*>(p + off1) : z;
     }
 }
 __device__ __forceinline__ void tile_store(char* tile, const TileRegs& t, int tid) {
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int q = tid + i * 256, row = q >> 3, c = q & 7;
-        *reinterpret_cast<u32x4*>(tile + row * KP + c * 16) = t.v[i];
-    }
+    const int off = (tid >> 3) * KP + (tid & 7) * 16;
+    *reinterpret_cast<u32x4*>(tile + off) = t.v[0];
+    *reinterpret_cast<u32x4*>(tile + off + 32 * KP) = t.v[1];
 }
 // 4 consecutive head-dim values of one row -> 8-byte store
 __device__ __forceinline__ void store4(floatX* p, float a, float b, float c, float d) {
@@ -343,8 +349,8 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
         else if (tid < 128) sD[buf][tid - 64] = rstat;
     };
     if (q_first < q_end) {
-        tile_load(rq, base, C3, 64 * q_first, T, tid);
-        tile_load(rdo, dobase, (size_t)C, 64 * q_first, T, tid);
+        tile_load(rq, base + (size_t)(64 * q_first) * C3, C3, T - (64 * q_first), tid);
+        tile_load(rdo, dobase + (size_t)(64 * q_first) * (size_t)C, (size_t)C, T - (64 * q_first), tid);
         load_stats(q_first);
         tile_store(sQ[0], rq, tid);
         tile_store(sdO[0], rdo, tid);
@@ -358,8 +364,8 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
         const char* tdo = sdO[buf];
         const bool more = qi + 1 < q_end;
         if (more) {
-            tile_load(rq, base, C3, 64 * (qi + 1), T, tid);
-            tile_load(rdo, dobase, (size_t)C, 64 * (qi + 1), T, tid);
+            tile_load(rq, base + (size_t)(64 * (qi + 1)) * C3, C3, T - (64 * (qi + 1)), tid);
+            tile_load(rdo, dobase + (size_t)(64 * (qi + 1)) * (size_t)C, (size_t)C, T - (64 * (qi + 1)), tid);
             load_stats(qi + 1);
         }
 #pragma unroll
@@ -466,8 +472,8 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
     const int last_q = min(qt * 128 + 127, T - 1);
     const int n_kt = last_q / 64 + 1;
     TileRegs rk, rv;
-    tile_load(rk, base + C, C3, 0, T, tid);
-    tile_load(rv, base + 2 * C, C3, 0, T, tid);
+    tile_load(rk, base + C + (size_t)(0) * C3, C3, T - (0), tid);
+    tile_load(rv, base + 2 * C + (size_t)(0) * C3, C3, T - (0), tid);
     tile_store(sK[0], rk, tid);
     tile_store(sV[0], rv, tid);
     __syncthreads();
@@ -477,8 +483,8 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
         const char* tv = sV[j & 1];
         const bool more = j + 1 < n_kt;
         if (more) {
-            tile_load(rk, base + C, C3, 64 * (j + 1), T, tid);
-            tile_load(rv, base + 2 * C, C3, 64 * (j + 1), T, tid);
+            tile_load(rk, base + C + (size_t)(64 * (j + 1)) * C3, C3, T - (64 * (j + 1)), tid);
+            tile_load(rv, base + 2 * C + (size_t)(64 * (j + 1)) * C3, C3, T - (64 * (j + 1)), tid);
         }
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
