@@ -32,7 +32,6 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 constexpr int HS = 64;
-constexpr int FA_FWD_WAVES = 4;       // waves (of 32 queries) per forward workgroup
 constexpr int KP = 144;               // LDS pitch (bytes) of a [row][64 x bf16] tile: 128 + 16, conflict-free for
                                       // both ds_read_b128 down a column of rows and the transposing 8-byte reads
 constexpr int TILE_BYTES = 64 * KP;   // 64 rows
@@ -100,6 +99,74 @@ __device__ __forceinline__ void store4(floatX* p, float a, float b, float c, flo
     *reinterpret_cast<bf16x4*>(p) = o;
 }
 
+// ---- tiles filled by direct-to-LDS loads ---------------------------------------------------------
+// A 64-row x 64-column bf16 tile stored without padding (128 B per row); the 16-byte chunk c of row r sits at chunk
+// c ^ swz(r). A direct-to-LDS load deposits a wave's 64 x 16 B linearly, so the swizzle is applied on the global
+// side (lane p of a row fetches chunk p ^ swz(row)). swz is chosen so that 16 consecutive rows read at one chunk
+// (MFMA operand along rows) and 4 rows x 32 B (transposing reads) both spread over all banks.
+constexpr int SW_TILE = 64 * 128;
+__device__ __forceinline__ int fa_swz(int row) { return (((row >> 1) & 3) << 1) | ((row >> 3) & 1); }
+typedef __attribute__((address_space(3))) void* fa_lds_ptr;
+struct FaLane {
+    unsigned rowb;          // frag along rows: byte offset of (row = lane%32, K step 0); step s is rowb ^ (s << 5)
+    unsigned colb0, colb1;  // transposing reads: byte offsets of this lane's two 8-byte pieces for (kbase 0, col0 0)
+    unsigned ld_off[2];     // staging: byte offset inside the global tile of this lane's 16 bytes of chunk i (row stride given at init)
+    __device__ __forceinline__ void init(int lane, int wave, size_t row_stride) {
+        const int idx = lane & 31, half = lane >> 5;
+        rowb = idx * 128 + ((half ^ fa_swz(idx)) << 4);
+        const int s16 = lane & 15, grp = lane >> 4;
+        const int r = 4 * (grp >> 1) + (s16 >> 2), col = (grp & 1) * 16 + 4 * (s16 & 3);
+        colb0 = r * 128 + (((col >> 3) ^ fa_swz(r)) << 4) + (col & 7) * 2;
+        colb1 = (r + 8) * 128 + (((col >> 3) ^ fa_swz(r + 8)) << 4) + (col & 7) * 2;
+#pragma unroll
+        for (int i = 0; i < 2; i++) {                     // a 4-wave workgroup: wave w deposits the 1 KiB chunks w and w + 4
+            const int row = (wave + 4 * i) * 8 + (lane >> 3), p = lane & 7;
+            ld_off[i] = (unsigned)((size_t)row * row_stride + ((p ^ fa_swz(row)) * 8)) * (unsigned)sizeof(floatX);
+        }
+    }
+};
+// Request this wave's two chunks of the tile whose first row is at `gtile` (all 64 rows must exist). The loads are
+// issued from inline asm, M0 (the LDS destination) included: when the compiler knows of a direct-to-LDS load in
+// flight it makes every later LDS read wait for it, whatever the read's address, which would turn the prefetch into
+// a synchronous copy. The kernel waits for its loads explicitly (fa_tiles_landed) before the barrier that publishes them.
+__device__ __forceinline__ void fa_tile_request(const FaLane& a, const floatX* gtile, unsigned lds_tile, int wave) {
+    const unsigned long long g = (unsigned long long)(size_t)gtile;
+    const unsigned dst = lds_tile + wave * 1024;
+    unsigned saved;
+    asm volatile("s_mov_b32 %0, m0\n\t"
+                 "s_mov_b32 m0, %1\n\t"
+                 "global_load_lds_dwordx4 %3, %2\n\t"
+                 "s_add_u32 m0, m0, 0x1000\n\t"
+                 "global_load_lds_dwordx4 %4, %2\n\t"
+                 "s_mov_b32 m0, %0"
+                 : "=&s"(saved) : "s"(dst), "s"(g), "v"(a.ld_off[0]), "v"(a.ld_off[1]) : "memory", "scc");
+}
+__device__ __forceinline__ void fa_tiles_landed() {
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // vmcnt(0), other counters untouched; as a builtin, so that the compiler also knows its own loads are done
+    asm volatile("" ::: "memory");
+}
+// LDS reads of these tiles go through integer addresses: a read the compiler can trace to the array that a
+// direct-to-LDS load is filling is preceded by a wait for every load in flight, which would undo the prefetch.
+__device__ __forceinline__ unsigned fa_lds_addr(const void* p) {
+    return (unsigned)(size_t)(__attribute__((address_space(3))) const char*)p;
+}
+__device__ __forceinline__ bf16x8 fa_frag_rows(unsigned tile, const FaLane& a, int row0, int s) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)(tile + row0 * 128 + (a.rowb ^ (unsigned)(s << 5))));
+}
+__device__ __forceinline__ f32x4 fa_lds_f32x4(unsigned addr) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>((size_t)addr);
+}
+// transposed operand of a swizzled tile (the order of frag_cols_accorder): two transposing 8-byte reads
+__device__ __forceinline__ bf16x8 fa_frag_cols(unsigned tile, const FaLane& a, int kbase, int col0) {
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+    const unsigned x = col0 ? 64u : 0u, t = tile + kbase * 128;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(t + (a.colb0 ^ x)));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(t + (a.colb1 ^ x)));
+    union { struct { s16x4 a, b; } s; bf16x8 v; } u;
+    u.s.a = lo; u.s.b = hi;
+    return u.v;
+}
+
 // Which (tile along T, batch*head) a workgroup works on. The grid is (tiles, B*NH) with x fastest, and workgroups
 // are dealt round-robin over the 8 XCDs, each with its own L2: taken literally, the tiles of one head would land
 // on 8 different XCDs and each would pull that head's K and V through its own L2. Instead XCD x takes the heads
@@ -121,7 +188,8 @@ __device__ __forceinline__ void fa_block_coords(int& tile, int& bh) {
 // two MFMAs that score takes part in), so everything else per score is kept to a minimum: the first MFMA of a
 // block starts from a constant zero instead of a cleared accumulator, maxima are taken three at a time, and the
 // K/V staging loads use a wave-uniform base with per-thread offsets that never change.
-template <int NWAVES = 8, int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no K/V streaming, 4: no barrier)
+// (Bringing K/V in by direct-to-LDS loads, as the dK/dV kernel does for Q/dO, measured 5 % slower here.)
+template <int NWAVES = 4, int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no K/V streaming, 4: no barrier)
 __global__ void __launch_bounds__(NWAVES * 64)
 fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
     __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
@@ -207,15 +275,17 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
         const char* tv = sV[(ABL & 2) ? 0 : (j & 1)];
         const bool more = j + 1 < n_kt && !(ABL & 2);
         if (more) stage_load(j + 1);
+        auto kfrag = [&](int row0, int s) -> bf16x8 { return frag_rows(tk, row0, s, lane); };
+        auto vfrag = [&](int kbase, int col0) -> bf16x8 { return frag_cols_accorder(tv, kbase, col0, lane); };
         if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
             // S^T for both 32-key blocks, the two accumulation chains interleaved
             f32x16 sacc[2];
-            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 0, 0, lane), qf[0], zero, 0, 0, 0);
-            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32, 0, lane), qf[0], zero, 0, 0, 0);
+            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, 0), qf[0], zero, 0, 0, 0);
+            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, 0), qf[0], zero, 0, 0, 0);
 #pragma unroll
             for (int s = 1; s < 4; s++) {
-                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 0, s, lane), qf[s], sacc[0], 0, 0, 0);
-                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tk, 32, s, lane), qf[s], sacc[1], 0, 0, 0);
+                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, s), qf[s], sacc[0], 0, 0, 0);
+                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, s), qf[s], sacc[1], 0, 0, 0);
             }
             if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
                 asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
@@ -252,7 +322,7 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
                 lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, lacc, 0, 0, 0);       // every row: sum over keys of P
 #pragma unroll
                 for (int d = 0; d < 2; d++)
-                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tv, 16 * s2, 32 * d, lane), pf, o[d], 0, 0, 0);
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(16 * s2, 32 * d), pf, o[d], 0, 0, 0);
             }
         }
         if (more) stage_store((j + 1) & 1);
@@ -299,6 +369,7 @@ fa_dot_do_o_kernel(float* __restrict__ D, const floatX* __restrict__ dout, const
 
 // ---- backward: dK, dV --------------------------------------------------------------------------------
 // grid (ceil(T/128), B*NH): wave w owns keys [128*kt + 32w, +32) and walks all later query tiles
+template <int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no Q/dO streaming, 4: no barrier)
 __global__ void __launch_bounds__(256)
 fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
                         const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
@@ -359,11 +430,11 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
     __syncthreads();
 
     for (int qi = q_first; qi < q_end; qi++) {
-        const int buf = (qi - q_first) & 1;
+        const int buf = (ABL & 2) ? 0 : (qi - q_first) & 1;
         const char* tq = sQ[buf];
         const char* tdo = sdO[buf];
-        const bool more = qi + 1 < q_end;
-        if (more) {
+        const bool more = qi + 1 < q_end && !(ABL & 2);
+        if (more && !(ABL & 16)) {
             tile_load(rq, base + (size_t)(64 * (qi + 1)) * C3, C3, T - (64 * (qi + 1)), tid);
             tile_load(rdo, dobase + (size_t)(64 * (qi + 1)) * (size_t)C, (size_t)C, T - (64 * (qi + 1)), tid);
             load_stats(qi + 1);
@@ -387,7 +458,7 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[buf][rr]);
                 d4[g] = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
 #pragma unroll
-                for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+                for (int e = 0; e < 4; e++) sacc[4 * g + e] = (ABL & 1) ? fmaf(sacc[4 * g + e], c, -l4[e]) : fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
             }
             if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
 #pragma unroll
@@ -410,12 +481,137 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 }
             }
         }
-        if (more) {
+        if (more && (ABL & 8)) {
+            asm volatile("" :: "v"(rq.v[0]), "v"(rq.v[1]), "v"(rdo.v[0]), "v"(rdo.v[1]), "v"(rstat));
+        } else if (more) {
             tile_store(sQ[buf ^ 1], rq, tid);
             tile_store(sdO[buf ^ 1], rdo, tid);
             store_stats(buf ^ 1);
         }
-        __syncthreads();
+        if (!(ABL & 4)) __syncthreads();
+    }
+
+    if (my_k < T) {
+        floatX* dkp = dqkv + ((size_t)b * T + my_k) * C3 + C + h * HS;
+        floatX* dvp = dqkv + ((size_t)b * T + my_k) * C3 + 2 * C + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int col = 32 * d + 8 * g + 4 * half;
+                store4(dkp + col, dk[d][4 * g] * 0.125f, dk[d][4 * g + 1] * 0.125f, dk[d][4 * g + 2] * 0.125f, dk[d][4 * g + 3] * 0.125f);
+                store4(dvp + col, dv[d][4 * g], dv[d][4 * g + 1], dv[d][4 * g + 2], dv[d][4 * g + 3]);
+            }
+    }
+}
+
+// Same computation with the Q / dO tiles brought in by direct-to-LDS loads (needs T % 64 == 0): no staging registers.
+template <int ABL = 0>
+__global__ void __launch_bounds__(256)
+fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                        const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+    __shared__ __attribute__((aligned(1024))) char sQ[2][SW_TILE];
+    __shared__ __attribute__((aligned(1024))) char sdO[2][SW_TILE];
+    extern __shared__ __attribute__((aligned(16))) float sStat[];   // [2][T]: log-sum-exp (in log2 units) and rowsum(dO*O) of every query of this head
+    float* sLall = sStat;
+    float* sDall = sStat + T;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    int kt, bh;
+    fa_block_coords(kt, bh);
+    const int b = bh / NH, h = bh % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const floatX* dobase = dout + (size_t)b * T * C + h * HS;
+    const float* lbase = stats + ((size_t)b * NH + h) * T;
+    const float* dbase = Dsum + ((size_t)b * NH + h) * T;
+    const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
+    const float c = 0.125f * LOG2E;
+
+    bf16x8 kf[4], vf[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_k < T) {
+            kf[s] = *reinterpret_cast<const bf16x8*>(base + C + (size_t)my_k * C3 + 16 * s + 8 * half);
+            vf[s] = *reinterpret_cast<const bf16x8*>(base + 2 * C + (size_t)my_k * C3 + 16 * s + 8 * half);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) { kf[s][e] = (__bf16)0.f; vf[s][e] = (__bf16)0.f; }
+        }
+    }
+    f32x16 dv[2], dk[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) { dv[d][r] = 0.f; dk[d][r] = 0.f; }
+
+    const int q_first = (kt * 128) / 64, q_end = CEIL_DIV(T, 64);
+    FaLane laq, lado;
+    laq.init(lane, __builtin_amdgcn_readfirstlane(wave), C3);
+    lado.init(lane, __builtin_amdgcn_readfirstlane(wave), (size_t)C);
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    // the per-query statistics of the whole head go to LDS once: no global loads besides the tiles inside the loop
+    for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = dbase[q]; }
+    if (q_first < q_end) {
+        fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
+        fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
+    }
+    fa_tiles_landed();
+    __syncthreads();
+
+    for (int qi = q_first; qi < q_end; qi++) {
+        const int buf = (ABL & 2) ? 0 : (qi - q_first) & 1;
+        const unsigned tq = fa_lds_addr(sQ[buf]), tdo = fa_lds_addr(sdO[buf]);
+        const unsigned stat_l = fa_lds_addr(sLall + 64 * qi), stat_d = fa_lds_addr(sDall + 64 * qi);
+        const bool more = qi + 1 < q_end && !(ABL & 2);
+        if (more) {
+            fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sQ[buf ^ 1]), uwave);
+            fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sdO[buf ^ 1]), uwave);
+        }
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            const int q0 = 64 * qi + 32 * qb;
+            if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
+            f32x16 sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
+            }
+            f32x4 d4[4];
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int rr = 32 * qb + g * 8 + half * 4;
+                const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
+                d4[g] = fa_lds_f32x4(stat_d + rr * 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) sacc[4 * g + e] = (ABL & 1) ? fmaf(sacc[4 * g + e], c, -l4[e]) : fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+            }
+            if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int q = q0 + acc_row(r, lane);
+                    if (q < my_k || q >= T) sacc[r] = 0.f;
+                }
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[g][e]);
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
+#pragma unroll
+                for (int d = 0; d < 2; d++) {
+                    dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
+                    dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tq, laq, 32 * qb + 16 * s2, 32 * d), dsf, dk[d], 0, 0, 0);
+                }
+            }
+        }
+        fa_tiles_landed();
+        if (!(ABL & 4)) __syncthreads();
     }
 
     if (my_k < T) {
@@ -643,7 +839,7 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 #if !defined(LLMK_FP32)
     LLMK_REQUIRE(hs == HS, "attention_forward: head size %d unsupported (bf16 build handles 64)", hs);
     LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
-    fa_forward_kernel<FA_FWD_WAVES><<<dim3(CEIL_DIV(T, 32 * FA_FWD_WAVES), B * NH), 64 * FA_FWD_WAVES, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+    fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
 #else
     LLMK_REQUIRE(hs <= 64, "attention_forward: head size %d unsupported (fp32 build handles <= 64)", hs);
     const size_t rows = (size_t)B * NH * T;
@@ -673,7 +869,10 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
     dim3 grid(CEIL_DIV(T, 128), B * NH);
     {   // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x here, 1.0x on dQ
         llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-        fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+        if (T % 64 == 0 && T <= 4096)       // whole tiles only, and 2*T floats of statistics in LDS beside the 32 KiB of tiles
+            fa_backward_dkdv_dma_kernel<><<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+        else
+            fa_backward_dkdv_kernel<><<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
         LAUNCH_CHECK();
     }
     llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
