@@ -179,6 +179,8 @@ gemm_pipelined_kernel(GemmArgs g) {
     };
 
     // --- per-thread load descriptors -----------------------------------------------------------
+    typedef __attribute__((address_space(3))) const char* lds_cptr;
+    const unsigned lds0 = (unsigned)(size_t)(lds_cptr)lds;                 // 1 KiB aligned
     // Each lane's 16 bytes of chunk i sit at (tile base of the operand) + voff[i]; the tile bases and the advance
     // per stage are wave-uniform, so a load costs one 32-bit VGPR of address.
     unsigned voff[CPW];          // byte offset of this lane's 16 bytes inside the operand's tile panel
@@ -217,22 +219,27 @@ gemm_pipelined_kernel(GemmArgs g) {
             }
         }
     };
+    // The loads are issued from inline asm, M0 (the LDS destination) included: when the compiler knows of a
+    // direct-to-LDS load in flight it makes every later LDS read it can see wait for ALL loads, e.g. the epilogue's
+    // strip reads for the next tile's first stages. All waiting for these loads is explicit (wait_vmcnt).
     auto issue = [&](int st, int buf) {
-        char* stage = lds + buf * STAGE;
         if (DBG & 1) return;
-        const char* pa = tile_base[0] + (size_t)st * stage_step[0];
-        const char* pb = tile_base[1] + (size_t)st * stage_step[1];
+        const unsigned stage = lds0 + buf * STAGE;
+        const unsigned long long pa = (unsigned long long)(size_t)(tile_base[0] + (size_t)st * stage_step[0]);
+        const unsigned long long pb = (unsigned long long)(size_t)(tile_base[1] + (size_t)st * stage_step[1]);
+        unsigned saved;
+        asm volatile("s_mov_b32 %0, m0" : "=s"(saved));
 #pragma unroll
         for (int i = 0; i < CPW; i++)
-            __builtin_amdgcn_global_load_lds((i * NW < A_CHUNKS ? pa : pb) + voff[i], (lds_void_ptr)(stage + lds_dst[i]), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2"
+                         :: "s"(stage + lds_dst[i]), "v"(voff[i]), "s"(i * NW < A_CHUNKS ? pa : pb) : "memory");
+        asm volatile("s_mov_b32 m0, %0" :: "s"(saved));
     };
 
     // --- MFMA operand reads ----------------------------------------------------------------------
     // One LDS address per 32-row fragment and lane, for K step 0 of buffer 0; the other steps and the other buffer
     // are reached by an XOR with the step (K-contiguous tiles: the swizzle is an XOR, so stepping the chunk index
     // commutes with it) or an immediate offset (K-major tiles), so the loop keeps TM + TN address registers.
-    typedef __attribute__((address_space(3))) const char* lds_cptr;
-    const unsigned lds0 = (unsigned)(size_t)(lds_cptr)lds;                 // 1 KiB aligned
     auto frag_base = [&](bool trans, int region, int rows, int row0) -> unsigned {
         if (!trans) {
             const int row = row0 + idx, f = (row >> 1) & 7;
