@@ -58,6 +58,12 @@ struct GemmArgs {
 
 #if !defined(LLMK_FP32)
 
+#ifndef LLMK_TR_ASM_BOTH
+#define LLMK_TR_ASM_BOTH 1
+#endif
+#ifndef LLMK_TR_ASM_MIXED
+#define LLMK_TR_ASM_MIXED 0
+#endif
 constexpr int PBK = 64;                 // K per stage
 constexpr int STAGES = 2;               // operand buffers: one being multiplied, one being filled
 constexpr int KGRAN = PBK;              // K (and the K range of a split) must be a multiple of this
@@ -128,6 +134,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int PASSES_OF_EPI = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
+    constexpr bool TR_ASM = (A_T && B_T) ? LLMK_TR_ASM_BOTH : LLMK_TR_ASM_MIXED;   // hand-issued or compiler-issued transposing reads
     constexpr int STRIP = 32 * 128;                            // epilogue staging per wave: 32 rows x 128 B
     constexpr int SPARE = (NW * STRIP + 1023) & ~1023;
     static_assert(STAGES * STAGE + SPARE <= LDS_TOTAL, "LDS budget");
@@ -266,8 +273,14 @@ gemm_pipelined_kernel(GemmArgs g) {
     // awaited by hand (await_frags below).
     auto frag_t = [&](unsigned base, auto off_lo, auto off_hi) -> bf16x8 {
         union { struct { s16x4 a, b; } s; bf16x8 v; } u;
-        u.s.a = ds_read_tr16<decltype(off_lo)::value>(base);
-        u.s.b = ds_read_tr16<decltype(off_hi)::value>(base);
+        if (TR_ASM) {
+            u.s.a = ds_read_tr16<decltype(off_lo)::value>(base);
+            u.s.b = ds_read_tr16<decltype(off_hi)::value>(base);
+        } else {
+            typedef s16x4 __attribute__((address_space(3))) * lp;
+            u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(size_t)(base + decltype(off_lo)::value));
+            u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lp)(size_t)(base + decltype(off_hi)::value));
+        }
         return u.v;
     };
 
@@ -302,6 +315,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     // to the wait so that nothing that uses them moves above it.
     constexpr int TR_READS = (A_T ? 2 * TM : 0) + (B_T ? 2 * TN : 0);       // hand-issued reads per 16-wide step
     auto await_frags = [&](bf16x8 (&fa)[TM], bf16x8 (&fb)[TN], auto younger) {
+        if (!TR_ASM) return;
         constexpr int Y = decltype(younger)::value;
         if (A_T) {
 #pragma unroll
