@@ -24,6 +24,14 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 METRIC = "train tokens/sec + MFU, GPT-2 124M bf16 B=64 T=1024, 1 MI355X"
 
+# Bytes per launch (read + written, averaged over the launches of a step) that the GEMM families move between L2 and
+# the memory side, from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over this same workload, scaled by what
+# the counters read for a copy kernel of known size (profiles/train_step_gpt2_124M_b64_t1024_hbm_traffic.txt has the
+# commands and the table). Valid for the default workload only. FETCH_SIZE counts L2 fills whether the Infinity Cache
+# or HBM served them.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemm_nn": 952091771, "gemm_tn_splitk": 848125171, "gemm_nt": 971393527,
+                                     "gemm_nt_gelu": 1250286793}
+
 # kernel families timed by the library -> roofline that bounds them
 MFMA_BOUND = {"gemm_nt", "gemm_nt_gelu", "gemm_nn", "gemm_nn_dgelu", "gemm_tn", "gemm_tn_splitk",
               "attention_forward", "attention_backward_dkdv", "attention_backward_dq"}
@@ -108,6 +116,7 @@ def main():
     L = pkg.load("bf16")           # raises if the HIP library is not built: there is no other path
     L.llmk_init(0)
     B, T = args.batch, args.seq
+    default_workload = (B, T, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 2)
     h = L.gpt2_create()
     L.gpt2_set_options(h, 1, args.recompute, args.gelu_fusion)
     L.gpt2_build_from_descriptor(h, args.model.encode())
@@ -146,7 +155,7 @@ def main():
             L.llmk_profile_get(i, name, C.byref(calls), C.byref(ms), C.byref(fl), C.byref(by))
             n = name.value.decode()
             rec = {"kernel": n, "launches_per_step": calls.value / nsteps, "ms_per_step": ms.value / nsteps,
-                   "avg_launch_ms": ms.value / max(calls.value, 1)}
+                   "avg_launch_ms": ms.value / max(calls.value, 1), "bytes_per_launch": by.value / max(calls.value, 1)}
             if n in MFMA_BOUND:
                 rec.update(bound="mfma", achieved=fl.value / (ms.value * 1e-3) / 1e12 if ms.value > 0 else 0.0,
                            peak=PEAK_BF16_TFLOPS, unit="TFLOP/s")
@@ -199,7 +208,9 @@ def main():
             kernels = timed
         d = timed[0]                           # the dominant family, timed live inside the timed steps
         roofline = {"kernel": d["kernel"], "bound": d["bound"], "achieved": d["achieved"], "peak": d["peak"],
-                    "unit": d["unit"], "frac": d["frac"], "traffic": None,
+                    "unit": d["unit"], "frac": d["frac"],
+                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(d["kernel"]) if default_workload else None,
+                    "algorithmic_bytes_per_launch": d["bytes_per_launch"],
                     "avg_launch_ms": d["avg_launch_ms"], "launches_per_step": d["launches_per_step"],
                     "ms_per_step": d["ms_per_step"]}
     L.gpt2_free(h)

@@ -189,7 +189,7 @@ __device__ __forceinline__ void fa_block_coords(int& tile, int& bh) {
 // block starts from a constant zero instead of a cleared accumulator, maxima are taken three at a time, and the
 // K/V staging loads use a wave-uniform base with per-thread offsets that never change.
 // (Bringing K/V in by direct-to-LDS loads, as the dK/dV kernel does for Q/dO, measured 5 % slower here.)
-template <int NWAVES = 4, int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no K/V streaming, 4: no barrier)
+template <int NWAVES = 4>
 __global__ void __launch_bounds__(NWAVES * 64)
 fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
     __shared__ __attribute__((aligned(16))) char sK[2][TILE_BYTES];
@@ -271,9 +271,9 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
     __syncthreads();
 
     for (int j = 0; j < n_kt; j++) {
-        const char* tk = sK[(ABL & 2) ? 0 : (j & 1)];
-        const char* tv = sV[(ABL & 2) ? 0 : (j & 1)];
-        const bool more = j + 1 < n_kt && !(ABL & 2);
+        const char* tk = sK[j & 1];
+        const char* tv = sV[j & 1];
+        const bool more = j + 1 < n_kt;
         if (more) stage_load(j + 1);
         auto kfrag = [&](int row0, int s) -> bf16x8 { return frag_rows(tk, row0, s, lane); };
         auto vfrag = [&](int kbase, int col0) -> bf16x8 { return frag_cols_accorder(tv, kbase, col0, lane); };
@@ -315,7 +315,7 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
             for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                 for (int r = 0; r < 16; r++)
-                    sacc[kb][r] = (ABL & 1) ? fmaf(sacc[kb][r], c, -m) : fast_exp2(fmaf(sacc[kb][r], c, -m));
+                    sacc[kb][r] = fast_exp2(fmaf(sacc[kb][r], c, -m));
 #pragma unroll
             for (int s2 = 0; s2 < 4; s2++) {
                 const bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
@@ -326,7 +326,7 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
             }
         }
         if (more) stage_store((j + 1) & 1);
-        if (!(ABL & 4)) __syncthreads();
+        __syncthreads();
     }
 
     const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
@@ -369,7 +369,6 @@ fa_dot_do_o_kernel(float* __restrict__ D, const floatX* __restrict__ dout, const
 
 // ---- backward: dK, dV --------------------------------------------------------------------------------
 // grid (ceil(T/128), B*NH): wave w owns keys [128*kt + 32w, +32) and walks all later query tiles
-template <int ABL = 0>   // ABL: measurement ablations (1: no exp, 2: no Q/dO streaming, 4: no barrier)
 __global__ void __launch_bounds__(256)
 fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
                         const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
@@ -430,11 +429,11 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
     __syncthreads();
 
     for (int qi = q_first; qi < q_end; qi++) {
-        const int buf = (ABL & 2) ? 0 : (qi - q_first) & 1;
+        const int buf = (qi - q_first) & 1;
         const char* tq = sQ[buf];
         const char* tdo = sdO[buf];
-        const bool more = qi + 1 < q_end && !(ABL & 2);
-        if (more && !(ABL & 16)) {
+        const bool more = qi + 1 < q_end;
+        if (more) {
             tile_load(rq, base + (size_t)(64 * (qi + 1)) * C3, C3, T - (64 * (qi + 1)), tid);
             tile_load(rdo, dobase + (size_t)(64 * (qi + 1)) * (size_t)C, (size_t)C, T - (64 * (qi + 1)), tid);
             load_stats(qi + 1);
@@ -458,7 +457,7 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[buf][rr]);
                 d4[g] = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
 #pragma unroll
-                for (int e = 0; e < 4; e++) sacc[4 * g + e] = (ABL & 1) ? fmaf(sacc[4 * g + e], c, -l4[e]) : fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+                for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
             }
             if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
 #pragma unroll
@@ -481,14 +480,12 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 }
             }
         }
-        if (more && (ABL & 8)) {
-            asm volatile("" :: "v"(rq.v[0]), "v"(rq.v[1]), "v"(rdo.v[0]), "v"(rdo.v[1]), "v"(rstat));
-        } else if (more) {
+        if (more) {
             tile_store(sQ[buf ^ 1], rq, tid);
             tile_store(sdO[buf ^ 1], rdo, tid);
             store_stats(buf ^ 1);
         }
-        if (!(ABL & 4)) __syncthreads();
+        __syncthreads();
     }
 
     if (my_k < T) {
@@ -506,7 +503,6 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
 }
 
 // Same computation with the Q / dO tiles brought in by direct-to-LDS loads (needs T % 64 == 0): no staging registers.
-template <int ABL = 0>
 __global__ void __launch_bounds__(256)
 fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
                         const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
@@ -560,10 +556,10 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
     __syncthreads();
 
     for (int qi = q_first; qi < q_end; qi++) {
-        const int buf = (ABL & 2) ? 0 : (qi - q_first) & 1;
+        const int buf = (qi - q_first) & 1;
         const unsigned tq = fa_lds_addr(sQ[buf]), tdo = fa_lds_addr(sdO[buf]);
         const unsigned stat_l = fa_lds_addr(sLall + 64 * qi), stat_d = fa_lds_addr(sDall + 64 * qi);
-        const bool more = qi + 1 < q_end && !(ABL & 2);
+        const bool more = qi + 1 < q_end;
         if (more) {
             fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sQ[buf ^ 1]), uwave);
             fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sdO[buf ^ 1]), uwave);
@@ -587,7 +583,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
                 d4[g] = fa_lds_f32x4(stat_d + rr * 4);
 #pragma unroll
-                for (int e = 0; e < 4; e++) sacc[4 * g + e] = (ABL & 1) ? fmaf(sacc[4 * g + e], c, -l4[e]) : fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+                for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
             }
             if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
 #pragma unroll
@@ -611,7 +607,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
             }
         }
         fa_tiles_landed();
-        if (!(ABL & 4)) __syncthreads();
+        __syncthreads();
     }
 
     if (my_k < T) {
@@ -870,9 +866,9 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
     {   // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x here, 1.0x on dQ
         llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
         if (T % 64 == 0 && T <= 4096)       // whole tiles only, and 2*T floats of statistics in LDS beside the 32 KiB of tiles
-            fa_backward_dkdv_dma_kernel<><<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
         else
-            fa_backward_dkdv_kernel<><<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
         LAUNCH_CHECK();
     }
     llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);

@@ -83,9 +83,7 @@ __device__ __forceinline__ void wait_vmcnt() {
 // Workgroup barrier WITHOUT the memory fence of __syncthreads(): the fence would wait for every outstanding
 // direct-to-LDS load (vmcnt(0)) and serialize the pipeline. Visibility of the K block that is about to be
 // read is established by the explicit vmcnt wait each wave does before arriving here.
-template <int DBG = 0>
 __device__ __forceinline__ void barrier_no_fence() {
-    if (DBG & 8) return;
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
@@ -93,9 +91,9 @@ __device__ __forceinline__ void barrier_no_fence() {
 
 // Output stores are non-temporal: a tile's output is not read again by this kernel, and a store that allocates in
 // L2 is acknowledged late enough (the waves count stores and loads with one counter) to hold up the next tile's loads.
-template <int DBG = 0, typename T>
+template <typename T>
 __device__ __forceinline__ void st_out(T* p, T v) {
-    if (DBG & 4096) *p = v; else __builtin_nontemporal_store(v, p);
+    __builtin_nontemporal_store(v, p);
 }
 // ... except where the next kernel reads a small result straight back (split-K partial sums, weight gradients)
 template <typename T>
@@ -123,11 +121,11 @@ __device__ __forceinline__ void tile_of(int t, int tiles_m, int tiles_n, int& tm
     tn = in_group / gsz;
 }
 
-template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI, int DBG = 0>   // DBG: measurement ablations (1: no loads, 2: no math, 4: no stores)
+template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
 __global__ void __launch_bounds__(WGM * WGN * 64)
 gemm_pipelined_kernel(GemmArgs g) {
 #if defined(__HIP_DEVICE_COMPILE__)   // device-only builtins below; the host pass only needs the launch stub
-    constexpr int NW = WGM * WGN, NT = NW * 64;
+    constexpr int NW = WGM * WGN;
     constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
     constexpr int A_STAGE = BM * PBK * 2, B_STAGE = BN * PBK * 2, STAGE = A_STAGE + B_STAGE;
     constexpr int A_CHUNKS = A_STAGE / 1024, B_CHUNKS = B_STAGE / 1024;
@@ -143,13 +141,6 @@ gemm_pipelined_kernel(GemmArgs g) {
     extern __shared__ __attribute__((aligned(1024))) char lds[];
 
     const int tid = threadIdx.x, lane = tid & 63;
-    if (DBG & 1) {   // ablation without loads: define the LDS contents (32: pseudo-random bits, else zeros)
-        for (int i = tid * 4; i < STAGES * STAGE + SPARE; i += NT * 4) {
-            unsigned v = (DBG & 32) ? ((squirrel_noise5((uint32_t)i, 17u) & 0x3fff3fffu) | 0x30003000u) : 0u;
-            *reinterpret_cast<unsigned*>(lds + i) = v;
-        }
-        __syncthreads();
-    }
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);     // scalar: LDS-DMA destinations must be wave-uniform
     const int wm = wave / WGN, wn = wave % WGN;
     // The two waves that share a SIMD (w and w + NW/2) request their share of a K block at different points of
@@ -230,7 +221,6 @@ gemm_pipelined_kernel(GemmArgs g) {
     // direct-to-LDS load in flight it makes every later LDS read it can see wait for ALL loads, e.g. the epilogue's
     // strip reads for the next tile's first stages. All waiting for these loads is explicit (wait_vmcnt).
     auto issue = [&](int st, int buf) {
-        if (DBG & 1) return;
         const unsigned stage = lds0 + buf * STAGE;
         const unsigned long long pa = (unsigned long long)(size_t)(tile_base[0] + (size_t)st * stage_step[0]);
         const unsigned long long pb = (unsigned long long)(size_t)(tile_base[1] + (size_t)st * stage_step[1]);
@@ -287,13 +277,6 @@ gemm_pipelined_kernel(GemmArgs g) {
     // fragments of the 16-wide K step S of the buffer at byte offset bufoff
     auto read_frags = [&](unsigned bufoff, auto sc, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
         constexpr int S = decltype(sc)::value;
-        if (DBG & 16) {
-#pragma unroll
-            for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
-#pragma unroll
-            for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
-            return;
-        }
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             if constexpr (A_T) fa[i] = frag_t(abase[i] + bufoff, std::integral_constant<int, S * 16 * BM * 2>{}, std::integral_constant<int, (S * 16 + 4) * BM * 2>{});
@@ -330,7 +313,6 @@ gemm_pipelined_kernel(GemmArgs g) {
     using NoneYounger = std::integral_constant<int, 0>;
     f32x16 acc[TM][TN];
     auto mma = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
-        if (DBG & 2) return;
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -365,7 +347,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr bool EPI_READS = (EPI == EPI_ACCUM);
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
-        if (!EPI_READS || (DBG & 4) || i >= TM) return;
+        if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
 #pragma unroll
         for (int pass = 0; pass < PASSES; pass++)
@@ -380,9 +362,6 @@ gemm_pipelined_kernel(GemmArgs g) {
                 }
     };
 
-    long long tc[8] = {0, 0, 0, 0, 0, 0, 0, 0};        // DBG & 128: cycle counts by phase (wave 0)
-    auto now = [&]() -> long long { return (DBG & 128) ? (long long)__builtin_readcyclecounter() : 0; };
-    const long long t_kernel = now();
 
     while (true) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
@@ -402,13 +381,9 @@ gemm_pipelined_kernel(GemmArgs g) {
         int next_m, next_n, next_split;
         const bool have_next = work_item(it + 1, next_m, next_n, next_split);
         auto buf_of = [&](int st) -> unsigned { return (unsigned)(st & 1) * STAGE; };
-        long long ta = now();
         if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
         else wait_vmcnt<0>();
-        barrier_no_fence<DBG>();                                  // stage 0 landed for everyone
-        long long tb = now();
-        tc[0] += tb - ta;
-        const long long t_loop = tb;
+        barrier_no_fence();                                       // stage 0 landed for everyone
         read_frags(buf_of(0), S0{}, fa0, fb0);
         for (int st = 0; st < nst - 1; st++) {
             const unsigned cur = buf_of(st);
@@ -423,11 +398,8 @@ gemm_pipelined_kernel(GemmArgs g) {
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
             __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
-            ta = now();
             if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
-            if (DBG & 128) { tb = now(); tc[6] += tb - ta; }
-            barrier_no_fence<DBG>();                              // ... and for everyone; the buffer of stage st is free
-            if (DBG & 128) { tb = now(); tc[2] += tb - ta; }
+            barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
             if (!late && st + 2 < nst) issue(st + 2, st & 1);
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
@@ -448,11 +420,9 @@ gemm_pipelined_kernel(GemmArgs g) {
             await_frags(fa1, fb1, NoneYounger{});
             mma(fa1, fb1);
         }
-        if (DBG & 128) { ta = now(); tc[3] += ta - t_loop; }
 
         // ---- request the next work item's first K blocks, then run the epilogue under them --------
-        barrier_no_fence<DBG>();                                  // every wave is done reading both buffers
-        if (DBG & 128) { tb = now(); tc[1] += tb - ta; }
+        barrier_no_fence();                                  // every wave is done reading both buffers
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
         prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
         it++;
@@ -468,7 +438,6 @@ gemm_pipelined_kernel(GemmArgs g) {
             issue(0, 0);
             if (next_nkb > 1) issue(1, 1);
         }
-        if (DBG & 128) { long long tcur = now(); tc[7] += tcur - tb; }
 
         // ---- epilogue ---------------------------------------------------------------------------------
         // Wave-private staging strip behind the operand buffers: 32 rows x 128 B, the 16-byte chunk c of row r stored
@@ -525,7 +494,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                         u32x4 raw = *reinterpret_cast<const u32x4*>(strip + row * 128 + ((ch ^ ((row >> 1) & 7)) << 4));
                         if (F32OUT) {
                             const int n = wn0 + pass * 32 + ch * 4;
-                            if (m < g.M && n < g.N && !(DBG & 4)) {
+                            if (m < g.M && n < g.N) {
                                 if (EPI == EPI_PARTIAL) {
                                     st_cached(reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n), raw);
                                 } else {
@@ -540,17 +509,17 @@ gemm_pipelined_kernel(GemmArgs g) {
                             }
                         } else {
                             const int n = wn0 + pass * 64 + ch * 8;
-                            if (m < g.M && n < g.N && !(DBG & 4)) {
+                            if (m < g.M && n < g.N) {
                                 const size_t o = (size_t)m * g.ldc + n;
                                 union { u32x4 u; bf16x8 h; } x, y;
                                 x.u = raw;
                                 if (EPI == EPI_BIAS_GELU) {
-                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.aux + o), x.u);
+                                    st_out(reinterpret_cast<u32x4*>(g.aux + o), x.u);
 #pragma unroll
                                     for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                 } else {
-                                    st_out<DBG>(reinterpret_cast<u32x4*>(g.C + o), x.u);
+                                    st_out(reinterpret_cast<u32x4*>(g.C + o), x.u);
                                 }
                             }
                         }
@@ -561,15 +530,9 @@ gemm_pipelined_kernel(GemmArgs g) {
                 prefetch_epilogue(cur_m0, cur_n0, i + 2);
             }
         }
-        if (DBG & 128) { tb = now(); tc[4] += tb - ta; }
         if (!have_next) break;
         st_young = cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
         nkb = next_nkb;
-    }
-    if ((DBG & 128) && lane == 0) {
-        tc[5] = now() - t_kernel;
-        long long* o = reinterpret_cast<long long*>(g.partial) + (blockIdx.x * NW + wave) * 8;
-        for (int i = 0; i < 8; i++) o[i] = tc[i];
     }
 #endif  // __HIP_DEVICE_COMPILE__
 }
