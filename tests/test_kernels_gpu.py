@@ -259,7 +259,9 @@ def run_matmul_forward(L, precision, x, w, b, pre_gelu, fusion):
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("M,Cc,OC,bias", [(64, 64, 64, True), (200, 72, 136, True), (256, 768, 2304, True),
                                            (512, 3072, 768, True), (128, 768, 50304, False),
-                                           (4096, 256, 4096, True), (4100, 192, 4360, False)])
+                                           (4096, 256, 4096, True), (4100, 192, 4360, False),
+                                           (4096, 1600, 4800, True),       # GPT-2 1558M qkv: 25 K stages, ragged N
+                                           (32768, 768, 2304, True)])      # enough row panels for the XCD-private work list
 def test_matmul_forward(precision, M, Cc, OC, bias):
     L = G.lib(precision)
     x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
@@ -292,7 +294,9 @@ def test_matmul_forward_gelu(precision, fusion, M, Cc, OC):
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("M,Cc,OC,bias", [(64, 64, 64, True), (200, 72, 136, True), (256, 768, 2304, True),
                                            (1024, 3072, 768, True), (8192, 768, 768, True), (4096, 2048, 2048, False),
-                                           (128, 256, 50304, False)])
+                                           (128, 256, 50304, False),
+                                           (32768, 768, 768, True),        # dinp on the 256x256 kernel with XCD-private row panels
+                                           (2048, 1600, 6400, True)])      # GPT-2 1558M fc
 def test_matmul_backward(precision, M, Cc, OC, bias):
     L = G.lib(precision)
     x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
