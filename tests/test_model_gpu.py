@@ -137,6 +137,33 @@ def test_fp32_small_model_vs_oracle_all_modes(recompute, gelu_fusion):
     m.free()
 
 
+@pytest.mark.parametrize("heads,channels", [(16, 1024), (25, 1600)])
+def test_wider_gpt2_layers_vs_oracle(heads, channels):
+    # the layer widths of GPT-2 350M (d24) and 1558M (d48), two layers deep with a small vocabulary so that the
+    # CPU oracle finishes in seconds: fp32 to the fp32 bar, bf16 to the bf16 bar. The learning rate keeps the loss of
+    # this one repeated batch of order 1 over the ten steps, where a relative bound on it means something
+    cfg = ol.Config(64, 2000, 2048, 2, heads, channels)
+    B, T = 2, 64
+    params = ol.init_params(cfg, 11)
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 17)
+    sizes, _ = ol.param_sizes(cfg)
+    ref = ol.cref_train(cfg, params, inp, tgt, B, T, 10, lr=2e-5, b1=0.9, b2=0.95, eps=1e-8, wd=0.1, wd_mask_2d=1,
+                        grad_clip=1.0, grad_step=0)
+    m = Model("fp32", cfg, B, T, params=params, master=0, recompute=1, gelu_fusion=2)
+    for s in range(10):
+        loss, norm = m.step(inp, tgt, s + 1, 2e-5, 0.9, 0.95, 1e-8, 0.1, clip=1.0)
+        assert abs(loss - ref["losses"][s]) <= 1e-5 * abs(ref["losses"][s]), (s, loss, ref["losses"][s])
+        if s == 0:
+            rel = per_tensor_rel(m.grads(), ref["grads"], sizes)
+            assert max(rel) <= 1e-3, dict(zip(NAMES, rel))
+    m.free()
+    m = Model("bf16", cfg, B, T, params=params, master=1, recompute=0, gelu_fusion=2)
+    for s in range(10):
+        loss, _ = m.step(inp, tgt, s + 1, 2e-5, 0.9, 0.95, 1e-8, 0.1, clip=1.0)
+        assert abs(loss - ref["losses"][s]) <= 2e-2, (s, loss, ref["losses"][s])
+    m.free()
+
+
 def gpt2_124m():
     return ol.Config(1024, 50257, 50304, 12, 12, 768)
 
