@@ -220,7 +220,9 @@ def main():
         "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"GPT-2 {args.model} ({nparams} params) full train step, bf16 + fp32 master weights/AdamW, "
-                               f"flash attention, clip 1.0 (BASELINE configs[2])",
+                               f"flash attention, clip 1.0" +
+                               {("d12", 64, 1024): " (BASELINE configs[2])", ("d24", 32, 1024): " (BASELINE configs[3])",
+                                ("d48", 16, 1024): " (BASELINE configs[4])"}.get((args.model, B, T), ""),
                    "global_batch": B, "seq_len": T, "tokens_per_step": B * T, "recompute": args.recompute,
                    "gelu_fusion": args.gelu_fusion, "parallelism": "single GPU"},
         "mfu": float(mfu), "mfu_peak_tflops": PEAK_BF16_TFLOPS,
