@@ -125,6 +125,15 @@ struct FaLane {
         }
     }
 };
+// A wave-uniform pointer, stated as such: pointer arithmetic that follows stays in scalar registers, which is where
+// fa_tile_request needs the tile address. (The builtin returns int: the halves are widened as unsigned.)
+template <typename T>
+__device__ __forceinline__ const T* fa_uniform(const T* p) {
+    const unsigned long long v = (unsigned long long)(size_t)p;
+    const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(v >> 32));
+    const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)v);
+    return reinterpret_cast<const T*>((size_t)(((unsigned long long)hi << 32) | (unsigned long long)lo));
+}
 // Request this wave's two chunks of the tile whose first row is at `gtile` (all 64 rows must exist). The loads are
 // issued from inline asm, M0 (the LDS destination) included: when the compiler knows of a direct-to-LDS load in
 // flight it makes every later LDS read wait for it, whatever the read's address, which would turn the prefetch into
@@ -188,7 +197,6 @@ __device__ __forceinline__ void fa_block_coords(int& tile, int& bh) {
 // two MFMAs that score takes part in), so everything else per score is kept to a minimum: the first MFMA of a
 // block starts from a constant zero instead of a cleared accumulator, maxima are taken three at a time, and the
 // K/V staging loads use a wave-uniform base with per-thread offsets that never change.
-// (Bringing K/V in by direct-to-LDS loads, as the dK/dV kernel does for Q/dO, measured 5 % slower here.)
 template <int NWAVES = 4>
 __global__ void __launch_bounds__(NWAVES * 64)
 fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
@@ -326,6 +334,135 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
             }
         }
         if (more) stage_store((j + 1) & 1);
+        __syncthreads();
+    }
+
+    const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
+    if (my_q < T) {
+        const float inv = 1.0f / l;
+        floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                store4(dst + 32 * d + 8 * g + 4 * half, o[d][4 * g] * inv, o[d][4 * g + 1] * inv, o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+        if (stats && half == 0) stats[((size_t)b * NH + h) * T + my_q] = (m + __log2f(l)) * 0.6931471805599453f;
+    }
+}
+
+// The same forward pass with K and V brought in by direct-to-LDS loads (T a multiple of 64: every tile is whole).
+// Without the staging registers the kernel fits 128 VGPRs, a fourth wave per SIMD, and with the loads issued from
+// inline asm the reads of the tile in use do not wait for the tile in flight. Same arithmetic in the same order as
+// fa_forward_kernel: the two give identical bits.
+__global__ void __launch_bounds__(256, 4)
+fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
+    constexpr int NWAVES = 4;
+    __shared__ __attribute__((aligned(1024))) char sK[2][SW_TILE];
+    __shared__ __attribute__((aligned(1024))) char sV[2][SW_TILE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    int tile_x, bh;
+    fa_block_coords(tile_x, bh);
+    const int qt = gridDim.x - 1 - tile_x;              // longest rows first
+    const int b = bh / NH, h = bh % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    constexpr int GQ = 32 * NWAVES;                       // queries per workgroup
+    const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
+    const float c = 0.125f * LOG2E;                       // 1/sqrt(64) folded into the exp2 argument
+
+    bf16x8 qf[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_q < T) qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+        else
+#pragma unroll
+            for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
+    }
+    f32x16 o[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[d][r] = 0.f;
+    float m = -INFINITY;
+    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    // The softmax denominator is accumulated by the matrix cores, which have cycles to spare here: a ones operand
+    // in place of V makes every row of this accumulator the sum over keys of the (bf16-rounded) probabilities of
+    // the lane's query - the same rounded values that multiply V.
+    f32x16 lacc = zero;
+    bf16x8 ones;
+#pragma unroll
+    for (int e = 0; e < 8; e++) ones[e] = (__bf16)1.0f;
+
+    const int last_q = min(qt * GQ + GQ - 1, T - 1);
+    const int n_kt = last_q / 64 + 1;
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    FaLane la;
+    la.init(lane, uwave, C3);
+    const floatX* kbase = fa_uniform(base + C);
+    const floatX* vbase = fa_uniform(base + 2 * C);
+    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
+    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
+    fa_tiles_landed();
+    __syncthreads();
+
+    for (int j = 0; j < n_kt; j++) {
+        const unsigned tk = fa_lds_addr(sK[j & 1]), tv = fa_lds_addr(sV[j & 1]);
+        if (j + 1 < n_kt) {                              // the other buffer was last read before the barrier that ended step j - 1
+            fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[(j + 1) & 1]), uwave);
+            fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[(j + 1) & 1]), uwave);
+        }
+        auto kfrag = [&](int row0, int s) -> bf16x8 { return fa_frag_rows(tk, la, row0, s); };
+        auto vfrag = [&](int kb, int col0) -> bf16x8 { return fa_frag_cols(tv, la, kb, col0); };
+        if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
+            // S^T for both 32-key blocks, the two accumulation chains interleaved
+            f32x16 sacc[2];
+            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, 0), qf[0], zero, 0, 0, 0);
+            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, 0), qf[0], zero, 0, 0, 0);
+#pragma unroll
+            for (int s = 1; s < 4; s++) {
+                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, s), qf[s], sacc[0], 0, 0, 0);
+                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, s), qf[s], sacc[1], 0, 0, 0);
+            }
+            if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
+                asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        if (64 * j + 32 * kb + acc_row(r, lane) > my_q) sacc[kb][r] = -INFINITY;
+            }
+            float mx = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+            for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
+            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            const float m_new = fmaxf(m, mx * c);
+            if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // some row's running max moved: rescale (rare after the first tiles)
+                asm volatile("" ::: "memory");
+                const float alpha = fast_exp2(m - m_new);
+                m = m_new;
+#pragma unroll
+                for (int r = 0; r < 16; r++) lacc[r] *= alpha;
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    sacc[kb][r] = fast_exp2(fmaf(sacc[kb][r], c, -m));
+#pragma unroll
+            for (int s2 = 0; s2 < 4; s2++) {
+                const bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
+                lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, lacc, 0, 0, 0);       // every row: sum over keys of P
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(16 * s2, 32 * d), pf, o[d], 0, 0, 0);
+            }
+        }
+        fa_tiles_landed();
         __syncthreads();
     }
 
@@ -724,6 +861,104 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
     }
 }
 
+// The same kernel with K and V brought in by direct-to-LDS loads (T a multiple of 64), like fa_forward_dma_kernel:
+// no staging registers, a fourth wave per SIMD, identical arithmetic.
+__global__ void __launch_bounds__(256, 4)
+fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                      const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+    __shared__ __attribute__((aligned(1024))) char sK[2][SW_TILE];
+    __shared__ __attribute__((aligned(1024))) char sV[2][SW_TILE];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
+    int tile_x, bh;
+    fa_block_coords(tile_x, bh);
+    const int qt = gridDim.x - 1 - tile_x;
+    const int b = bh / NH, h = bh % NH;
+    const int C = NH * HS;
+    const size_t C3 = 3 * (size_t)C;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+    const float c = 0.125f * LOG2E;
+
+    bf16x8 qf[4], dof[4];
+#pragma unroll
+    for (int s = 0; s < 4; s++) {
+        if (my_q < T) {
+            qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+            dof[s] = *reinterpret_cast<const bf16x8*>(dout + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) { qf[s][e] = (__bf16)0.f; dof[s][e] = (__bf16)0.f; }
+        }
+    }
+    const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
+    const float dsum = my_q < T ? Dsum[((size_t)b * NH + h) * T + my_q] : 0.f;
+    f32x16 dq[2];
+#pragma unroll
+    for (int d = 0; d < 2; d++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) dq[d][r] = 0.f;
+
+    const int last_q = min(qt * 128 + 127, T - 1);
+    const int n_kt = last_q / 64 + 1;
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    FaLane la;
+    la.init(lane, uwave, C3);
+    const floatX* kbase = fa_uniform(base + C);
+    const floatX* vbase = fa_uniform(base + 2 * C);
+    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
+    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
+    fa_tiles_landed();
+    __syncthreads();
+
+    for (int j = 0; j < n_kt; j++) {
+        const unsigned tk = fa_lds_addr(sK[j & 1]), tv = fa_lds_addr(sV[j & 1]);
+        if (j + 1 < n_kt) {                              // the other buffer was last read before the barrier that ended step j - 1
+            fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[(j + 1) & 1]), uwave);
+            fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[(j + 1) & 1]), uwave);
+        }
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            const int k0 = 64 * j + 32 * kb;
+            if (k0 > qw0 + 31) continue;
+            f32x16 sacc, pacc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 4; s++) {
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
+            if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    if (k0 + acc_row(r, lane) > my_q) sacc[r] = 0.f;
+            }
+#pragma unroll
+            for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const bf16x8 dsf = pack_acc(pacc, s2);
+#pragma unroll
+                for (int d = 0; d < 2; d++)
+                    dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
+            }
+        }
+        fa_tiles_landed();
+        __syncthreads();
+    }
+    if (my_q < T) {
+        floatX* dqp = dqkv + ((size_t)b * T + my_q) * C3 + h * HS;
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+                store4(dqp + 32 * d + 8 * g + 4 * half, dq[d][4 * g] * 0.125f, dq[d][4 * g + 1] * 0.125f, dq[d][4 * g + 2] * 0.125f,
+                       dq[d][4 * g + 3] * 0.125f);
+    }
+}
+
 #else
 // =============================================================================================
 // fp32 build: one wavefront per row, lanes = head dimensions (hs <= 64)
@@ -835,7 +1070,10 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 #if !defined(LLMK_FP32)
     LLMK_REQUIRE(hs == HS, "attention_forward: head size %d unsupported (bf16 build handles 64)", hs);
     LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
-    fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+    if (T % 64 == 0)
+        fa_forward_dma_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+    else
+        fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
 #else
     LLMK_REQUIRE(hs <= 64, "attention_forward: head size %d unsupported (fp32 build handles <= 64)", hs);
     const size_t rows = (size_t)B * NH * T;
@@ -872,7 +1110,10 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
         LAUNCH_CHECK();
     }
     llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
-    fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+    if (T % 64 == 0)
+        fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+    else
+        fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
     LAUNCH_CHECK();
 #else
     LLMK_REQUIRE(hs <= 64, "attention_backward: head size %d unsupported (fp32 build handles <= 64)", hs);
