@@ -862,10 +862,11 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
 }
 
 // The same kernel with K and V brought in by direct-to-LDS loads (T a multiple of 64), like fa_forward_dma_kernel:
-// no staging registers, a fourth wave per SIMD, identical arithmetic.
+// no staging registers, a fourth wave per SIMD. It also produces D = rowsum(dO * O) itself and writes it out,
+// which takes the place of fa_dot_do_o_kernel's pass over dO and O: it runs before the dK/dV kernel.
 __global__ void __launch_bounds__(256, 4)
 fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
-                      const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+                          const floatX* __restrict__ o, const float* __restrict__ stats, float* __restrict__ Dsum, int T, int NH) {
     __shared__ __attribute__((aligned(1024))) char sK[2][SW_TILE];
     __shared__ __attribute__((aligned(1024))) char sV[2][SW_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
@@ -891,7 +892,19 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
         }
     }
     const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
-    const float dsum = my_q < T ? Dsum[((size_t)b * NH + h) * T + my_q] : 0.f;
+    // D = rowsum(dO * O) of the lane's query from the dO values it already holds: the two halves of the wave own
+    // 32 head dimensions each. The dK/dV kernel, launched after this one, reads D from memory.
+    float dsum = 0.f;
+    if (my_q < T) {
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            const bf16x8 of = *reinterpret_cast<const bf16x8*>(o + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
+#pragma unroll
+            for (int e = 0; e < 8; e++) dsum = fmaf((float)dof[s][e], (float)of[e], dsum);
+        }
+    }
+    dsum += __shfl_xor(dsum, 32, WAVE);
+    if (my_q < T && half == 0) Dsum[((size_t)b * NH + h) * T + my_q] = dsum;
     f32x16 dq[2];
 #pragma unroll
     for (int d = 0; d < 2; d++)
@@ -1095,26 +1108,35 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
     float* Dsum = (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
     const size_t nrows = (size_t)B * T * NH;
     const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
-    {
-        llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
-        fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
-        LAUNCH_CHECK();
-    }
-    dim3 grid(CEIL_DIV(T, 128), B * NH);
-    {   // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x here, 1.0x on dQ
+    const dim3 grid(CEIL_DIV(T, 128), B * NH);
+    // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x on dK/dV, 1.0x on dQ
+    if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
+        {
+            llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+            fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
+            LAUNCH_CHECK();
+        }
         llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-        if (T % 64 == 0 && T <= 4096)       // whole tiles only, and 2*T floats of statistics in LDS beside the 32 KiB of tiles
+        if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
             fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
         else
             fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
         LAUNCH_CHECK();
-    }
-    llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
-    if (T % 64 == 0)
-        fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-    else
+    } else {
+        {
+            llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
+            fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
+            LAUNCH_CHECK();
+        }
+        {
+            llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+            fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            LAUNCH_CHECK();
+        }
+        llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
         fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-    LAUNCH_CHECK();
+        LAUNCH_CHECK();
+    }
 #else
     LLMK_REQUIRE(hs <= 64, "attention_backward: head size %d unsupported (fp32 build handles <= 64)", hs);
     const size_t rows = (size_t)B * NH * T;
