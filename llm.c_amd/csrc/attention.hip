@@ -367,6 +367,14 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
     const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    // the first K and V tiles are requested before anything else: they travel while the wave fetches its own rows
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    FaLane la;
+    la.init(lane, uwave, C3);
+    const floatX* kbase = fa_uniform(base + C);
+    const floatX* vbase = fa_uniform(base + 2 * C);
+    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
+    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
     constexpr int GQ = 32 * NWAVES;                       // queries per workgroup
     const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
     const float c = 0.125f * LOG2E;                       // 1/sqrt(64) folded into the exp2 argument
@@ -396,13 +404,6 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
 
     const int last_q = min(qt * GQ + GQ - 1, T - 1);
     const int n_kt = last_q / 64 + 1;
-    const int uwave = __builtin_amdgcn_readfirstlane(wave);
-    FaLane la;
-    la.init(lane, uwave, C3);
-    const floatX* kbase = fa_uniform(base + C);
-    const floatX* vbase = fa_uniform(base + 2 * C);
-    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
-    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
     fa_tiles_landed();
     __syncthreads();
 
@@ -654,12 +655,24 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
     const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
-    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * HS;      // reassigned below, stated uniform
     const floatX* dobase = dout + (size_t)b * T * C + h * HS;
     const float* lbase = stats + ((size_t)b * NH + h) * T;
     const float* dbase = Dsum + ((size_t)b * NH + h) * T;
     const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
     const float c = 0.125f * LOG2E;
+    // the first Q and dO tiles are requested before anything else: they travel while the wave fetches its own rows
+    const int q_first = (kt * 128) / 64, q_end = CEIL_DIV(T, 64);
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    FaLane laq, lado;
+    laq.init(lane, uwave, C3);
+    lado.init(lane, uwave, (size_t)C);
+    base = fa_uniform(base);
+    dobase = fa_uniform(dobase);
+    if (q_first < q_end) {
+        fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
+        fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
+    }
 
     bf16x8 kf[4], vf[4];
 #pragma unroll
@@ -678,17 +691,8 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
 #pragma unroll
         for (int r = 0; r < 16; r++) { dv[d][r] = 0.f; dk[d][r] = 0.f; }
 
-    const int q_first = (kt * 128) / 64, q_end = CEIL_DIV(T, 64);
-    FaLane laq, lado;
-    laq.init(lane, __builtin_amdgcn_readfirstlane(wave), C3);
-    lado.init(lane, __builtin_amdgcn_readfirstlane(wave), (size_t)C);
-    const int uwave = __builtin_amdgcn_readfirstlane(wave);
     // the per-query statistics of the whole head go to LDS once: no global loads besides the tiles inside the loop
     for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = dbase[q]; }
-    if (q_first < q_end) {
-        fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
-        fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
-    }
     fa_tiles_landed();
     __syncthreads();
 
@@ -877,6 +881,14 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
     const floatX* base = qkv + (size_t)b * T * C3 + h * HS;
+    // the first K and V tiles are requested before anything else: they travel while the wave fetches its own rows
+    const int uwave = __builtin_amdgcn_readfirstlane(wave);
+    FaLane la;
+    la.init(lane, uwave, C3);
+    const floatX* kbase = fa_uniform(base + C);
+    const floatX* vbase = fa_uniform(base + 2 * C);
+    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
+    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
     const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
     const float c = 0.125f * LOG2E;
 
@@ -913,13 +925,6 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
 
     const int last_q = min(qt * 128 + 127, T - 1);
     const int n_kt = last_q / 64 + 1;
-    const int uwave = __builtin_amdgcn_readfirstlane(wave);
-    FaLane la;
-    la.init(lane, uwave, C3);
-    const floatX* kbase = fa_uniform(base + C);
-    const floatX* vbase = fa_uniform(base + 2 * C);
-    fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
-    fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
     fa_tiles_landed();
     __syncthreads();
 
