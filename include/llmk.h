@@ -62,6 +62,11 @@ void llmk_profile_reset(void);
 int llmk_profile_count(void);
 void llmk_profile_get(int i, char* name64, int* calls, double* ms, double* flops, double* bytes);
 
+/* Zero `bytes` bytes at `ptr` on `stream`: the cudaMemsetAsync calls of the training step (gradients and losses,
+ * train_gpt2.cu:800-801; the residual-stream gradient, train_gpt2.cu:828) as a store kernel that runs at HBM write
+ * bandwidth. Any alignment and size. */
+void llmk_zero(void* ptr, size_t bytes, void* stream);
+
 /* ---- encoder (llmc/encoder.cuh) ---------------------------------------------------------- */
 
 /* encoder_forward, llmc/encoder.cuh:157. out[b,t,:] = wte[inp[b,t],:] + wpe[t,:] */

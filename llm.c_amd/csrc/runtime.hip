@@ -2,6 +2,7 @@
 // Counterpart of the reference's common_start / cudaCheck / cublaslt_workspace
 // (train_gpt2.cu:1173-1200, llmc/cuda_common.h:52-58, llmc/cublas_common.h:28-31).
 #include "common.hpp"
+#include <algorithm>
 #include "../../include/llmk.h"
 #include <cstdarg>
 #include <cstring>
@@ -104,6 +105,17 @@ static void prof_collect() {
 
 }  // namespace llmk
 
+namespace {
+// 16-byte non-temporal zero stores, a few workgroups per CU striding the buffer
+__global__ void __launch_bounds__(256) zero_kernel(float* __restrict__ p, size_t nvec) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    const f4 z = {0.f, 0.f, 0.f, 0.f};
+    const size_t stride = (size_t)gridDim.x * 256;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += stride)
+        __builtin_nontemporal_store(z, reinterpret_cast<f4*>(p) + i);
+}
+}  // namespace
+
 extern "C" {
 
 void llmk_profile_enable(int on) { llmk::prof_collect(); llmk::g_prof_on = on != 0; }
@@ -144,5 +156,21 @@ void llmk_device_props(int* num_cu, int* max_threads_per_cu, char* name256) {
 void llmk_set_error_mode(int record) { llmk::g_error_mode = record ? 1 : 0; }
 const char* llmk_last_error(void) { return llmk::g_last_error.c_str(); }
 void llmk_clear_error(void) { llmk::g_last_error.clear(); llmk::g_failed = false; }
+
+void llmk_zero(void* ptr, size_t bytes, void* stream) {
+    if (llmk::failed() || bytes == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    const size_t head = (16 - (uintptr_t)ptr % 16) % 16;          // bytes before the first 16-byte boundary
+    if (bytes < head + 16) { HIP_CHECK(hipMemsetAsync(ptr, 0, bytes, st)); return; }
+    char* p = (char*)ptr;
+    if (head) HIP_CHECK(hipMemsetAsync(p, 0, head, st));
+    const size_t nvec = (bytes - head) / 16, tail = bytes - head - nvec * 16;
+    llmk::ProfScope prof("zero", 0, (double)nvec * 16, st);
+    const size_t want = (nvec + 255) / 256;
+    const unsigned grid = (unsigned)std::min(want, (size_t)llmk::device_info().num_cu * 16);
+    zero_kernel<<<grid, 256, 0, st>>>((float*)(p + head), nvec);
+    LAUNCH_CHECK();
+    if (tail) HIP_CHECK(hipMemsetAsync(p + head + nvec * 16, 0, tail, st));
+}
 
 }  // extern "C"

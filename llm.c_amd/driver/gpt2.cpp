@@ -473,7 +473,7 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
                  L = m->config.num_layers, NH = m->config.num_heads, C = m->config.channels, X = m->X;
     if (micro_step == 0) {
         hipCheck(hipMemsetAsync(m->acts.losses, 0, B * T * sizeof(float), st));
-        hipCheck(hipMemsetAsync(m->grads_memory, 0, m->num_parameters * X, st));
+        llmk_zero(m->grads_memory, m->num_parameters * X, st);
     }
     ParameterTensors p = m->params, g = m->grads;
     ActivationTensors a = m->acts;
@@ -485,7 +485,7 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
     llmk_fused_classifier(a.output, a.losses, dloss, m->targets, (int)B, (int)T, (int)V, (int)Vp, 1, st);
 
     xptr dresidual = a.scratch_btc;
-    hipCheck(hipMemsetAsync(dresidual, 0, B * T * C * X, st));
+    llmk_zero(dresidual, B * T * C * X, st);
     float* scratchF = (float*)a.output;
 
     llmk_matmul_backward(a.scratch_bt4c, g.wte, nullptr, a.output, a.lnf, p.wte, nullptr, (int)B, (int)T, (int)C, (int)Vp, st, nullptr, 1);

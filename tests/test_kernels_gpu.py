@@ -169,6 +169,18 @@ def test_gelu(precision):
     close(G.host(d_g), rd, **tol(precision, 1e-5, bf16_atol=1e-2))
 
 
+@pytest.mark.parametrize("offset,nbytes", [(0, 0), (0, 16), (3, 5), (5, 11), (1, 64), (16, 4096), (7, 100003), (0, 50 * 1024 * 1024 + 9)])
+def test_zero_touches_exactly_its_range(offset, nbytes):
+    # any alignment and size: head and tail bytes around the 16-byte store kernel, neighbours left alone
+    L = G.lib("bf16")
+    total = offset + nbytes + 64
+    base = (np.arange(total) % 251 + 1).astype(np.uint8)
+    d = G.dev(base)
+    L.llmk_zero(CT.c_void_p(d.data_ptr() + offset), nbytes, None)
+    want = base.copy(); want[offset:offset + nbytes] = 0
+    np.testing.assert_array_equal(G.host(d), want)
+
+
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("N,OC", [(37, 64), (300, 3072), (2048, 264)])
 def test_gelu_backward_bias_equals_the_two_separate_steps(precision, N, OC):
