@@ -1,0 +1,195 @@
+"""Per-kernel microbenchmark at GPT-2 124M shapes (N = B*T = 65536 rows, bf16 storage, fp32 accumulation),
+in the manner of the reference's dev/cuda/*.cu programs (timing loop dev/cuda/common.h:350-385: a cache flush
+before every repetition, device events around the launch).
+
+Every case is called through the C ABI (include/llmk.h); the library brackets each of its kernel launches with HIP
+events on the launch stream (llmk_profile_*), so a case that launches several kernels (matmul_backward: dinp GEMM,
+dweight GEMM, split-K reduce, bias gradient) reports each of them. Inputs are N(0,1) from a fixed seed, weights
+N(0,0.02). Before each repetition 1 GiB is overwritten, which evicts the 8 x 4 MiB L2s and the 256 MiB Infinity Cache.
+
+    python llm.c_amd/microbench.py [--reps 20] [--only gemm,attention,...] [--json out.json]
+
+Prints, per kernel family and case: median and minimum milliseconds, the algorithmic TFLOP/s or GB/s at the median,
+and the fraction of the roofline that bounds the family (2500 TFLOP/s bf16 MFMA, 8000 GB/s HBM). PyTorch is used
+for device memory and random numbers only.
+"""
+import argparse
+import ctypes as C
+import importlib.util
+import json
+import os
+import statistics
+import sys
+
+import numpy as np
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+spec = importlib.util.spec_from_file_location("llmc_amd", os.path.join(HERE, "__init__.py"))
+pkg = importlib.util.module_from_spec(spec)
+sys.modules["llmc_amd"] = pkg
+spec.loader.exec_module(pkg)
+
+PEAK_TFLOPS, PEAK_GBS = 2500.0, 8000.0
+MFMA_FAMILIES = ("gemm", "attention_forward", "attention_backward_dq", "attention_backward_dkdv")
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--only", default="")
+    ap.add_argument("--json", default="")
+    args = ap.parse_args()
+    only = [s for s in args.only.split(",") if s]
+
+    L = pkg.load("bf16")          # raises LibraryMissing when the HIP library has not been built
+    L.llmk_init(0)
+    dev = "cuda"
+    p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
+    g = torch.Generator(device=dev); g.manual_seed(1234)
+    randn = lambda *shape, scale=1.0: (torch.randn(*shape, device=dev, generator=g) * scale).bfloat16()
+    flush_buf = torch.empty(1 << 30, dtype=torch.uint8, device=dev)
+
+    name = C.create_string_buffer(64)
+    calls, ms, fl, by = C.c_int(), C.c_double(), C.c_double(), C.c_double()
+
+    def measure(fn, prepare=None):
+        """-> {family: (list of ms per rep, flops per rep, bytes per rep, launches per rep)}"""
+        out = {}
+        fn(); torch.cuda.synchronize()                        # warm-up (workspace growth, attribute setting)
+        for _ in range(args.reps):
+            if prepare: prepare()
+            flush_buf.zero_(); torch.cuda.synchronize()
+            L.llmk_profile_reset(); L.llmk_profile_enable(1)
+            fn()
+            torch.cuda.synchronize(); L.llmk_profile_enable(0)
+            for i in range(L.llmk_profile_count()):
+                L.llmk_profile_get(i, name, C.byref(calls), C.byref(ms), C.byref(fl), C.byref(by))
+                rec = out.setdefault(name.value.decode(), ([], fl.value, by.value, calls.value))
+                rec[0].append(ms.value)
+        return out
+
+    results = []
+
+    def report(case, out):
+        for fam, (times, flops, nbytes, ncalls) in out.items():
+            med, mn = statistics.median(times), min(times)
+            mfma = fam.startswith(MFMA_FAMILIES)
+            if mfma:
+                rate, unit, frac = flops / med * 1e-9, "TFLOP/s", flops / med * 1e-9 / PEAK_TFLOPS
+            else:
+                rate, unit, frac = nbytes / med * 1e-6, "GB/s", nbytes / med * 1e-6 / PEAK_GBS
+            print(f"{case:34s} {fam:26s} x{ncalls:<2d} median {med:8.4f} ms  min {mn:8.4f} ms  {rate:9.1f} {unit:8s} {100 * frac:5.1f} % of {'MFMA' if mfma else 'HBM'} peak",
+                  flush=True)
+            results.append({"case": case, "kernel": fam, "launches": ncalls, "median_ms": med, "min_ms": mn, "rate": rate, "unit": unit,
+                            "bound": "mfma" if mfma else "hbm", "frac": frac, "flops": flops, "bytes": nbytes})
+
+    def want(tag):
+        return not only or any(o in tag for o in only)
+
+    B, T, Cc, NH, V, Vp, NL = 64, 1024, 768, 12, 50257, 50304, 12
+    N = B * T
+
+    if want("gemm"):
+        for nm, K, OC in [("qkv", 768, 2304), ("attproj", 768, 768), ("fc", 768, 3072), ("fcproj", 3072, 768), ("lm_head", 768, 50304)]:
+            inp, w = randn(N, K), randn(OC, K, scale=0.02)
+            bias = None if nm == "lm_head" else randn(OC, scale=0.02)
+            out_t = torch.empty(N, OC, device=dev, dtype=torch.bfloat16)
+            report(f"matmul_forward {nm} K={K} OC={OC}",
+                   measure(lambda: L.llmk_matmul_forward(p(out_t), p(inp), p(w), p(bias), B, T, K, OC, None, None, 0)))
+            if nm == "fc":
+                pre = torch.empty_like(out_t)
+                report(f"matmul_forward+gelu {nm} K={K} OC={OC}",
+                       measure(lambda: L.llmk_matmul_forward(p(out_t), p(inp), p(w), p(bias), B, T, K, OC, None, p(pre), 2)))
+                del pre
+            dout = out_t.normal_(generator=g)                  # reuse the output buffer as the upstream gradient
+            dinp, dw = torch.empty_like(inp), torch.zeros_like(w)
+            dbias = None if bias is None else torch.zeros_like(bias)
+            scratch = torch.empty(max(L.llmk_matmul_backward_bias_scratch_floats(OC), 1), device=dev, dtype=torch.float32)
+            report(f"matmul_backward {nm} K={K} OC={OC}",
+                   measure(lambda: L.llmk_matmul_backward(p(dinp), p(dw), p(dbias), p(dout), p(inp), p(w), p(scratch), B, T, K, OC, None, None, 0)))
+            del inp, w, out_t, dout, dinp, dw, scratch
+            torch.cuda.empty_cache()
+
+    if want("layernorm"):
+        x, y = randn(N, Cc), randn(N, Cc)
+        w, b = randn(Cc), randn(Cc)
+        o, r = torch.empty_like(x), torch.empty_like(x)
+        mean, rstd = torch.empty(N, device=dev), torch.empty(N, device=dev)
+        report("layernorm_forward 65536x768", measure(lambda: L.llmk_layernorm_forward(p(o), p(mean), p(rstd), p(x), p(w), p(b), B, T, Cc, None)))
+        report("fused_residual_forward5 65536x768",
+               measure(lambda: L.llmk_fused_residual_forward5(p(r), p(o), p(mean), p(rstd), p(x), p(y), p(w), p(b), N, Cc, None)))
+        dinp, dw, db = torch.zeros_like(x), torch.zeros_like(w), torch.zeros_like(b)
+        scratch = torch.empty(L.llmk_layernorm_backward_scratch_floats(Cc), device=dev, dtype=torch.float32)
+        report("layernorm_backward 65536x768",
+               measure(lambda: L.llmk_layernorm_backward(p(dinp), p(dw), p(db), p(scratch), p(y), p(x), p(w), p(mean), p(rstd), B, T, Cc, None)))
+        del x, y, o, r, dinp
+
+    if want("gelu"):
+        n = N * 4 * Cc
+        x, o = randn(N, 4 * Cc), torch.empty(N, 4 * Cc, device=dev, dtype=torch.bfloat16)
+        report("gelu_forward 65536x3072", measure(lambda: L.llmk_gelu_forward(p(o), p(x), n, None)))
+        report("gelu_backward_inplace 65536x3072", measure(lambda: L.llmk_gelu_backward_inplace(p(o), p(x), n, None)))
+        db = torch.zeros(4 * Cc, device=dev, dtype=torch.bfloat16)
+        scratch = torch.empty(max(L.llmk_matmul_backward_bias_scratch_floats(4 * Cc), 1), device=dev, dtype=torch.float32)
+        report("gelu_backward_bias 65536x3072", measure(lambda: L.llmk_gelu_backward_bias(p(o), p(x), p(db), p(scratch), B, T, 4 * Cc, None)))
+        del x, o
+
+    if want("encoder"):
+        tok = torch.randint(0, V, (N,), device=dev, dtype=torch.int32, generator=g)
+        tok_host = np.ascontiguousarray(tok.cpu().numpy())
+        wte, wpe = randn(Vp, Cc, scale=0.02), randn(T, Cc, scale=0.02)
+        o = torch.empty(N, Cc, device=dev, dtype=torch.bfloat16)
+        report("encoder_forward 65536x768", measure(lambda: L.llmk_encoder_forward(p(o), p(tok), p(wte), p(wpe), B, T, Cc, None)))
+        dout = randn(N, Cc)
+        dwte, dwpe = torch.zeros_like(wte), torch.zeros_like(wpe)
+        ncg = -(-Cc // 512)
+        scratch = torch.zeros(N * ncg * 20 + 64, dtype=torch.uint8, device=dev)
+        wl, bk = np.zeros(N * ncg, np.int32), np.zeros(4 * N * ncg, np.int32)
+        report("encoder_backward 65536x768 (device kernels; the host bucket sort is not in these figures)",
+               measure(lambda: L.llmk_encoder_backward(p(dwte), p(dwpe), p(scratch), wl.ctypes.data_as(C.c_void_p), bk.ctypes.data_as(C.c_void_p),
+                                                       p(dout), p(tok), tok_host.ctypes.data_as(C.c_void_p), B, T, Cc, 42, None)))
+        del wte, dwte, o, dout
+
+    if want("classifier"):
+        logits = torch.empty(N, Vp, device=dev, dtype=torch.bfloat16)
+        src = randn(2048, Vp)
+        tgt = torch.randint(0, V, (N,), device=dev, dtype=torch.int32, generator=g)
+        losses = torch.zeros(N, device=dev)
+
+        def refill():                                           # the kernel works in place: give it logits again
+            for i in range(0, N, 2048):
+                logits[i:i + 2048].copy_(src)
+        report("fused_classifier 65536x50304", measure(lambda: L.llmk_fused_classifier(p(logits), p(losses), 1.0 / N, p(tgt), B, T, V, Vp, 1, None), prepare=refill))
+        del logits, src
+        torch.cuda.empty_cache()
+
+    if want("adamw"):
+        P = 124475904
+        params, grads = randn(P, scale=0.02), randn(P, scale=0.01)
+        master = params.float()
+        m, v = torch.zeros(P, device=dev), torch.zeros(P, device=dev)
+        report("adamw_update 124475904 params",
+               measure(lambda: L.llmk_adamw_update(p(params), p(master), p(grads), p(m), p(v), P, 0, 0, 0, 1, 6e-4, 0.9, 0.95, 1, 1e-8, 0.1, 1.0, 7, None)))
+        nb = C.c_int(1)
+        maxb = L.llmk_get_max_num_block_sums(C.byref(nb), 1)
+        partial = torch.zeros(maxb, device=dev)
+        report("global_norm_squared 124475904 grads", measure(lambda: L.llmk_global_norm_squared(p(partial), p(grads), P, 0, 1, maxb, 1, None)))
+        del params, grads, master, m, v
+
+    if want("attention"):
+        qkv = randn(B, T, 3 * Cc, scale=0.5)
+        o = torch.empty(B, T, Cc, device=dev, dtype=torch.bfloat16)
+        stats = torch.empty(B * NH * T, device=dev)
+        report("attention_forward B64 NH12 T1024 hs64", measure(lambda: L.llmk_attention_forward(p(o), p(stats), p(qkv), B, T, NH, Cc, None)))
+        dout, dqkv = randn(B, T, Cc, scale=0.1), torch.empty_like(qkv)
+        report("attention_backward B64 NH12 T1024 hs64",
+               measure(lambda: L.llmk_attention_backward(p(dqkv), p(dout), p(qkv), p(o), p(stats), B, T, NH, Cc, None)))
+
+    if args.json:
+        with open(args.json, "w") as f:
+            json.dump({"reps": args.reps, "peak_tflops": PEAK_TFLOPS, "peak_gbs": PEAK_GBS, "results": results}, f, indent=1)
+
+
+if __name__ == "__main__":
+    main()
