@@ -369,7 +369,7 @@ def attention_case(precision, B, T, NH, seed=0):
 
 
 @pytest.mark.parametrize("precision", PRECS)
-@pytest.mark.parametrize("B,T,NH", [(2, 64, 2), (1, 128, 3), (2, 200, 2), (1, 1, 2), (1, 1024, 2), (2, 384, 12)])
+@pytest.mark.parametrize("B,T,NH", [(2, 64, 2), (1, 128, 3), (2, 200, 2), (1, 1, 2), (1, 1024, 2), (2, 384, 12), (4, 192, 2), (1, 320, 3)])
 def test_attention_forward_backward(precision, B, T, NH):
     L = G.lib(precision)
     qkv, g, ro, rlse, rd, Cc = attention_case(precision, B, T, NH)
