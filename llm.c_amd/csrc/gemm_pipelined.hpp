@@ -184,10 +184,14 @@ gemm_pipelined_kernel(GemmArgs g) {
     unsigned voff[CPW];          // byte offset of this lane's 16 bytes inside the operand's tile panel
     int lds_dst[CPW];            // wave-uniform byte offset of the chunk inside a stage
     const char* tile_base[2];    // A and B panels of the current work item at its first K
+    const char* tile_base_n[2];  // ... of the next work item, when its first stage is requested before the current one ends
     size_t stage_step[2];        // bytes to advance per stage
+    auto bases_into = [&](const char* (&tb)[2], int m0, int n0, int kbeg) {
+        tb[0] = reinterpret_cast<const char*>(A_T ? g.A + (size_t)kbeg * g.lda + m0 : g.A + (size_t)m0 * g.lda + kbeg);
+        tb[1] = reinterpret_cast<const char*>(B_T ? g.B + (size_t)kbeg * g.ldb + n0 : g.B + (size_t)n0 * g.ldb + kbeg);
+    };
     auto setup_bases = [&](int m0, int n0, int kbeg) {
-        tile_base[0] = reinterpret_cast<const char*>(A_T ? g.A + (size_t)kbeg * g.lda + m0 : g.A + (size_t)m0 * g.lda + kbeg);
-        tile_base[1] = reinterpret_cast<const char*>(B_T ? g.B + (size_t)kbeg * g.ldb + n0 : g.B + (size_t)n0 * g.ldb + kbeg);
+        bases_into(tile_base, m0, n0, kbeg);
         stage_step[0] = (A_T ? (size_t)PBK * g.lda : (size_t)PBK) * sizeof(floatX);
         stage_step[1] = (B_T ? (size_t)PBK * g.ldb : (size_t)PBK) * sizeof(floatX);
     };
@@ -220,10 +224,10 @@ gemm_pipelined_kernel(GemmArgs g) {
     // The loads are issued from inline asm, M0 (the LDS destination) included: when the compiler knows of a
     // direct-to-LDS load in flight it makes every later LDS read it can see wait for ALL loads, e.g. the epilogue's
     // strip reads for the next tile's first stages. All waiting for these loads is explicit (wait_vmcnt).
-    auto issue = [&](int st, int buf) {
+    auto issue_from = [&](const char* const (&tb)[2], int st, int buf) {
         const unsigned stage = lds0 + buf * STAGE;
-        const unsigned long long pa = (unsigned long long)(size_t)(tile_base[0] + (size_t)st * stage_step[0]);
-        const unsigned long long pb = (unsigned long long)(size_t)(tile_base[1] + (size_t)st * stage_step[1]);
+        const unsigned long long pa = (unsigned long long)(size_t)(tb[0] + (size_t)st * stage_step[0]);
+        const unsigned long long pb = (unsigned long long)(size_t)(tb[1] + (size_t)st * stage_step[1]);
         unsigned saved;
         asm volatile("s_mov_b32 %0, m0" : "=s"(saved));
 #pragma unroll
@@ -232,6 +236,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                          :: "s"(stage + lds_dst[i]), "v"(voff[i]), "s"(i * NW < A_CHUNKS ? pa : pb) : "memory");
         asm volatile("s_mov_b32 m0, %0" :: "s"(saved));
     };
+    auto issue = [&](int st, int buf) { issue_from(tile_base, st, buf); };
 
     // --- MFMA operand reads ----------------------------------------------------------------------
     // One LDS address per 32-row fragment and lane, for K step 0 of buffer 0; the other steps and the other buffer
@@ -381,6 +386,22 @@ gemm_pipelined_kernel(GemmArgs g) {
         int next_m, next_n, next_split;
         const bool have_next = work_item(it + 1, next_m, next_n, next_split);
         auto buf_of = [&](int st) -> unsigned { return (unsigned)(st & 1) * STAGE; };
+        // With an even number of stages the last-but-one stage frees buffer 0, which is where the next work item's
+        // first stage belongs: it is requested there and then, a stage before the tile ends, instead of at the tile
+        // change (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
+        // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
+        // short of scalar registers).
+        constexpr bool EARLY0 = EPI != EPI_ACCUM && EPI != EPI_PARTIAL;
+        int next_kbeg = 0, next_nkb = 0;
+        bool early0 = false;
+        if (have_next) {
+            next_kbeg = next_split * g.k_per_split;
+            next_nkb = (min(g.K, next_kbeg + g.k_per_split) - next_kbeg) / PBK;
+            if constexpr (EARLY0) {
+                early0 = nst >= 2 && (nst & 1) == 0 && !voff_edge && !is_edge(next_m, next_n);
+                if (early0) bases_into(tile_base_n, next_m * BM, next_n * BN, next_kbeg);
+            }
+        }
         if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
         else wait_vmcnt<0>();
         barrier_no_fence();                                       // stage 0 landed for everyone
@@ -400,7 +421,10 @@ gemm_pipelined_kernel(GemmArgs g) {
             __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
             if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
             barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
-            if (!late && st + 2 < nst) issue(st + 2, st & 1);
+            if (!late) {
+                if (st + 2 < nst) issue(st + 2, st & 1);
+                else if (EARLY0 && early0) issue_from(tile_base_n, 0, 0);
+            }
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
@@ -411,6 +435,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
+            if (EARLY0 && late && early0) issue_from(tile_base_n, 0, 0);
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
@@ -426,16 +451,18 @@ gemm_pipelined_kernel(GemmArgs g) {
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
         prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
         it++;
-        int next_nkb = 0;
         if (have_next) {
             tile_m = next_m; tile_n = next_n; split = next_split;
-            kbeg = split * g.k_per_split;
-            next_nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
-            setup_bases(tile_m * BM, tile_n * BN, kbeg);
-            const bool edge = is_edge(tile_m, tile_n);
-            if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
-            voff_edge = edge;
-            issue(0, 0);
+            kbeg = next_kbeg;
+            if (EARLY0 && early0) {                               // its first stage is already on the way
+                tile_base[0] = tile_base_n[0]; tile_base[1] = tile_base_n[1];
+            } else {
+                setup_bases(tile_m * BM, tile_n * BN, kbeg);
+                const bool edge = is_edge(tile_m, tile_n);
+                if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
+                voff_edge = edge;
+                issue(0, 0);
+            }
             if (next_nkb > 1) issue(1, 1);
         }
 
