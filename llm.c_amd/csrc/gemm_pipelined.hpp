@@ -340,6 +340,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     bool voff_edge = is_edge(tile_m, tile_n);
     setup_bases(tile_m * BM, tile_n * BN, kbeg);
     setup_voff(tile_m * BM, tile_n * BN);
+    int par = 0;                        // stage s of the current work item lives in buffer (s + par) & 1
     issue(0, 0);
     if (nkb > 1) issue(1, 1);
     bool st_young = false;              // the previous epilogue's stores are all issued and counted
@@ -379,16 +380,17 @@ gemm_pipelined_kernel(GemmArgs g) {
 
         // ---- K loop over stages of 64, software-pipelined: the operands of the next 16-wide step (and the
         // barrier that publishes the next stage) are requested while the matrix cores work on the current step.
-        // Stage s lives in buffer s & 1; while it is multiplied, stage s+1 is in flight.
+        // Stage s lives in buffer (s + par) & 1; while it is multiplied, stage s+1 is in flight.
         bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
         const int nst = nkb;
         // the next work item's coordinates are worked out here (integer divisions), under the K loop's MFMAs
         int next_m, next_n, next_split;
         const bool have_next = work_item(it + 1, next_m, next_n, next_split);
-        auto buf_of = [&](int st) -> unsigned { return (unsigned)(st & 1) * STAGE; };
-        // With an even number of stages the last-but-one stage frees buffer 0, which is where the next work item's
-        // first stage belongs: it is requested there and then, a stage before the tile ends, instead of at the tile
-        // change (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
+        auto buf_idx = [&](int st) -> int { return (st + par) & 1; };
+        auto buf_of = [&](int st) -> unsigned { return (unsigned)buf_idx(st) * STAGE; };
+        // The last-but-one stage frees a buffer a whole stage before the tile ends: the next work item's first stage
+        // is requested into it there and then instead of at the tile change, and the next item's stages alternate
+        // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
         constexpr bool EARLY0 = EPI != EPI_ACCUM && EPI != EPI_PARTIAL;
@@ -398,7 +400,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             next_kbeg = next_split * g.k_per_split;
             next_nkb = (min(g.K, next_kbeg + g.k_per_split) - next_kbeg) / PBK;
             if constexpr (EARLY0) {
-                early0 = nst >= 2 && (nst & 1) == 0 && !voff_edge && !is_edge(next_m, next_n);
+                early0 = nst >= 2 && !voff_edge && !is_edge(next_m, next_n);
                 if (early0) bases_into(tile_base_n, next_m * BM, next_n * BN, next_kbeg);
             }
         }
@@ -411,7 +413,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            if (late && st >= 1) issue(st + 1, (st + 1) & 1);
+            if (late && st >= 1) issue(st + 1, buf_idx(st + 1));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
@@ -422,8 +424,8 @@ gemm_pipelined_kernel(GemmArgs g) {
             if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
             barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
             if (!late) {
-                if (st + 2 < nst) issue(st + 2, st & 1);
-                else if (EARLY0 && early0) issue_from(tile_base_n, 0, 0);
+                if (st + 2 < nst) issue(st + 2, buf_idx(st));
+                else if (EARLY0 && early0) issue_from(tile_base_n, 0, buf_idx(st));
             }
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
@@ -435,7 +437,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            if (EARLY0 && late && early0) issue_from(tile_base_n, 0, 0);
+            if (EARLY0 && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
@@ -454,16 +456,18 @@ gemm_pipelined_kernel(GemmArgs g) {
         if (have_next) {
             tile_m = next_m; tile_n = next_n; split = next_split;
             kbeg = next_kbeg;
-            if (EARLY0 && early0) {                               // its first stage is already on the way
+            if (EARLY0 && early0) {                               // its first stage is already on the way, in the buffer of stage nst-2
                 tile_base[0] = tile_base_n[0]; tile_base[1] = tile_base_n[1];
+                par = (nst - 2 + par) & 1;
             } else {
                 setup_bases(tile_m * BM, tile_n * BN, kbeg);
                 const bool edge = is_edge(tile_m, tile_n);
                 if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
                 voff_edge = edge;
+                par = 0;
                 issue(0, 0);
             }
-            if (next_nkb > 1) issue(1, 1);
+            if (next_nkb > 1) issue(1, (1 + par) & 1);
         }
 
         // ---- epilogue ---------------------------------------------------------------------------------

@@ -308,7 +308,9 @@ def test_matmul_forward_gelu(precision, fusion, M, Cc, OC):
                                            (1024, 3072, 768, True), (8192, 768, 768, True), (4096, 2048, 2048, False),
                                            (128, 256, 50304, False),
                                            (32768, 768, 768, True),        # dinp on the 256x256 kernel with XCD-private row panels
-                                           (2048, 1600, 6400, True)])      # GPT-2 1558M fc
+                                           (2048, 1600, 6400, True),       # GPT-2 1558M fc
+                                           (4096, 1600, 1600, True),       # odd number of 64-wide K stages in dinp
+                                           (16384, 832, 1600, False)])     # odd stage counts on the 256x256 kernel
 def test_matmul_backward(precision, M, Cc, OC, bias):
     L = G.lib(precision)
     x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
