@@ -369,6 +369,39 @@ gemm_pipelined_kernel(GemmArgs g) {
     };
 
 
+    // Bias of the wave's columns (EPI_BIAS, EPI_BIAS_GELU), fetched once per tile near its end: block j, quad q holds
+    // the four columns j*32 + 8q + 4*half + 0..3 of the wave tile, the ones the lane owns in the epilogue. Loads that
+    // the compiler issues are awaited with vmcnt(0), which also waits for every hand-issued tile load in flight; so
+    // they are placed in the one window in which this wave has none: from the start of the tile's last stage (the
+    // last-but-one stage ended with a wait for everything) until the wave requests the next tile's first stage, which
+    // these kernels do only after claiming the bias (bias_ready), half-way through the last stage. Tiles that reach past N take plain
+    // loads in the epilogue instead (the columns are tested there).
+    constexpr bool HAS_BIAS = (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU);
+    bf16x4 biasv[HAS_BIAS ? TN : 1][4];
+    bool bias_fast = false;
+    auto request_bias = [&](int n0) {
+        if constexpr (HAS_BIAS) {
+            bias_fast = g.bias != nullptr && n0 + BN <= g.N;
+            // unconditional, so that the values stay in the registers they arrive in (a branch here makes the compiler
+            // copy them where the paths join, which needs them at once): without a usable bias the lanes read the
+            // first bytes of A, which are there, and the epilogue ignores what they got
+            const floatX* bp = bias_fast ? g.bias + n0 + wn * WTN + 4 * half : g.A + 4 * half;
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) biasv[j][q] = *reinterpret_cast<const bf16x4*>(bp + j * 32 + q * 8);
+            asm volatile("" ::: "memory");                        // the loads stay here: nothing below may pull them down to their use
+        }
+    };
+    auto bias_ready = [&]() {
+        if constexpr (HAS_BIAS) {
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) asm volatile("" : "+v"(biasv[j][q]));
+        }
+    };
+
     while (true) {
         const int m0 = tile_m * BM, n0 = tile_n * BN;
 #pragma unroll
@@ -425,7 +458,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
             if (!late) {
                 if (st + 2 < nst) issue(st + 2, buf_idx(st));
-                else if (EARLY0 && early0) issue_from(tile_base_n, 0, buf_idx(st));
+                else if (EARLY0 && !HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(st));
             }
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
@@ -433,14 +466,17 @@ gemm_pipelined_kernel(GemmArgs g) {
         }
         {
             const unsigned cur = buf_of(nst - 1);
+            request_bias(n0);                                     // nothing of this wave is in flight here (kernels with a bias)
             prefetch_epilogue(m0, n0, 0);
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
-            if (EARLY0 && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
+            if (EARLY0 && !HAS_BIAS && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1);
+            bias_ready();                                         // two 16-wide steps after the request
+            if (EARLY0 && HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
             read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0);
@@ -493,7 +529,11 @@ gemm_pipelined_kernel(GemmArgs g) {
                             float v[4];
 #pragma unroll
                             for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
-                            if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+                            if (HAS_BIAS && bias_fast) {
+                                const bf16x4 b4 = biasv[HAS_BIAS ? j : 0][q];
+#pragma unroll
+                                for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
+                            } else if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
                                 if (g.bias) {
                                     const int n = wn0 + nl;
                                     if (n < g.N) {
