@@ -184,8 +184,9 @@ residual_kernel(floatX* __restrict__ out, const floatX* __restrict__ a, const fl
 // partial goes to scratch[block][2][C]; a second kernel adds the partials in block order, so
 // the result does not depend on scheduling (no atomics).
 // One workgroup per CU, as many waves as the accumulators leave room for: 12 (three per SIMD) up to NV = 2, where the
-// kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8, then 4 beyond.
-constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 4 ? 8 : 4; }
+// kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8 at NV = 3,
+// 4 beyond (at NV = 4, C = 1600, eight waves spill half of their accumulators).
+constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 3 ? 8 : 4; }
 template <int NV>
 __global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : 1)
 ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
