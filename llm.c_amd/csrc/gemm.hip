@@ -266,6 +266,9 @@ bool pipelined_ok(const GemmArgs& g) {
     return g.K % KGRAN == 0 && g.k_per_split % KGRAN == 0 && g.lda % 8 == 0 && g.ldb % 8 == 0 && g.ldc % 8 == 0 &&
            g.N % 8 == 0 && al(g.A, 16) && al(g.B, 16) && al(g.C, 16) && (!g.bias || al(g.bias, 8)) && (!g.aux || al(g.aux, 16));
 }
+// The pipelined kernel's += epilogue spills registers (it holds the old values of a whole tile); with it available,
+// a single "split" written as fp32 partials and folded in by the reduce pass is 30 % faster than accumulating in place.
+bool tn_partial_always(const GemmArgs& g) { return pipelined_ok(g); }
 template <int BM, int BN, int WGM, int WGN, bool A_T, bool B_T, int EPI>
 void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
     constexpr int NW = WGM * WGN;
@@ -419,6 +422,7 @@ constexpr int K_ALIGN = 4;
 constexpr int BIG_TILE = 128, SMALL_TILE = 128, K_STEP = 16;
 template <bool A_T, bool B_T, int EPI>
 void launch_best(const GemmArgs& g, int splits, bool big, hipStream_t st) { launch_gemm<A_T, B_T, EPI>(g, splits, big, st); }
+bool tn_partial_always(const GemmArgs&) { return false; }
 #endif
 
 // C[m][n] (+)= sum over splits of partial[s][m][n], in split order
@@ -643,15 +647,17 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         const size_t tiles_small = (size_t)CEIL_DIV(OC, SMALL_TILE) * CEIL_DIV(C, SMALL_TILE);
         const bool big = tiles_big >= 8;                          // split-K fills the machine when there are few big tiles
         const size_t tiles = big ? tiles_big : tiles_small;
-        int splits = (int)max((size_t)1, (size_t)num_cu / tiles);
-        if (tiles > (size_t)num_cu) {
-            // More tiles than CUs: the last round of a persistent launch may be mostly empty (591 tiles on 256 CUs
-            // run as 3 rounds at 77 %). Splitting K by a small factor evens the rounds out; each extra split costs
-            // one fp32 pass over the output, priced here at 2 % of the GEMM.
+        // Split K so that the work items fill whole rounds of the persistent launch (27 tiles -> 9 splits = 243 items on
+        // 256 CUs; 591 tiles -> 3 splits, 1773 items = 6.9 rounds instead of 3 rounds at 77 %; 175 tiles -> 4 splits).
+        // Each split costs one fp32 pass over the output (8 bytes per element written and read back, against 2*M flop
+        // per element in the GEMM): 800/M of the GEMM's time at the rates measured, 1.2 % at M = 65536.
+        int splits = 1;
+        {
             double best = 1e30;
-            for (int s = 1; s <= 4; s++) {
+            const double pass = 800.0 / (double)M;
+            for (int s = 1; s <= 32; s++) {
                 const size_t work = tiles * s, rounds = CEIL_DIV(work, (size_t)num_cu);
-                const double cost = (double)(rounds * num_cu) / (double)work + (s > 1 ? 0.02 * s : 0.0);
+                const double cost = (double)(rounds * num_cu) / (double)work + pass * s;
                 if (cost < best) { best = cost; splits = s; }
             }
         }
@@ -661,7 +667,7 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         splits = CEIL_DIV(ksteps, steps_per);
         g.k_per_split = steps_per * K_STEP;
         const double tn_bytes = ((double)M * OC + (double)M * C + 2.0 * OC * C) * sizeof(floatX);
-        if (splits == 1) {
+        if (splits == 1 && !tn_partial_always(g)) {
             llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
             launch_best<true, true, EPI_ACCUM>(g, 1, big, st);
         } else {
