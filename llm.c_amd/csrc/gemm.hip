@@ -563,7 +563,8 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
         llmk_gelu_forward(out, pre_gelu, M * OC, stream);
     } else {
         g.C = (floatX*)out;
-        launch_best<false, false, EPI_BIAS>(g, 1, big, st);
+        if (bias) launch_best<false, false, EPI_BIAS>(g, 1, big, st);
+        else launch_best<false, false, EPI_STORE>(g, 1, big, st);     // the LM head: no bias to fetch, no window to keep for it
     }
 }
 
