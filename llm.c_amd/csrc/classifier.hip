@@ -19,71 +19,112 @@ __device__ __forceinline__ float cls_exp(float x) { return expf(x); }
 __device__ __forceinline__ float cls_exp(float x) { return __expf(x); }
 #endif
 
+// exp(x - mx) as the two passes below evaluate it. bf16 build: one fma and one hardware exp2 with the 1/ln2
+// folded into both operands (mxl = mx * log2(e)); fp32 build: the library expf of the difference.
+#if defined(LLMK_FP32)
+__device__ __forceinline__ float cls_exp_rel(float x, float mx, float) { return expf(x - mx); }
+__device__ __forceinline__ float cls_scaled(float e, float inv, float dloss, float) { return e * inv * dloss; }
+#else
+__device__ __forceinline__ float cls_exp_rel(float x, float, float mxl) { return __builtin_amdgcn_exp2f(fmaf(x, 1.4426950408889634f, -mxl)); }
+__device__ __forceinline__ float cls_scaled(float e, float, float, float inv_dloss) { return e * inv_dloss; }
+#endif
+
 // NVT: 16-byte vectors held per lane; requires P/VN <= NVT*CLS_BLOCK.
+// The vectors whose VN columns are all real ([0, V/VN)) take loops without any per-element test; the one vector
+// that straddles V (when V is not a multiple of VN) is held by a single lane and handled on the side, and the
+// target column is patched in the one vector that holds it. Per element that leaves: max; fma, exp2, add; and
+// fma, exp2, multiply, convert.
 template <int NVT, bool WRITE>
-__global__ void __launch_bounds__(CLS_BLOCK)
+__global__ void __launch_bounds__(CLS_BLOCK, NVT <= 7 ? 8 : 4)   // up to 7 vectors: 64 registers, two workgroups (rows) per CU
 fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses, float dloss,
                         const int* __restrict__ targets, int V, int P) {
     __shared__ float red[2][16];
     const int64_t row = (int64_t)gridDim.x - 1 - blockIdx.x;
     floatX* x = logits + row * (int64_t)P;
-    const int nvec = P / VN;               // vectors that hold at least one of the V real columns:
-    const int nvalid = CEIL_DIV(V, VN);    // [0, nvalid); the rest is padding and is never touched
+    const int nfull = V / VN, rem = V - nfull * VN;     // padding columns [V, P) are never touched
     const int tid = threadIdx.x;
     const int target = targets[row];
+    const int tvec = target / VN, tk = target - tvec * VN;
+    const bool edge = rem != 0 && tid == nfull % CLS_BLOCK;   // this lane holds the straddling vector
 
-    vecX r[NVT];
+    vecX r[NVT], re;
     float mx = -INFINITY;
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        int v = tid + i * CLS_BLOCK;
-        if (v < nvalid) {
+        const int v = tid + i * CLS_BLOCK;
+        if (v < nfull) {
             r[i] = ld_vec(x + (size_t)v * VN);
 #pragma unroll
-            for (int k = 0; k < VN; k++)
-                if (v * VN + k < V) mx = fmaxf(mx, to_f32(r[i][k]));
+            for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
         }
     }
-    (void)nvec;
+    if (edge) {
+        re = ld_vec(x + (size_t)nfull * VN);
+#pragma unroll
+        for (int k = 0; k < VN; k++)
+            if (k < rem) mx = fmaxf(mx, to_f32(re[k]));
+    }
     mx = block_reduce<true>(mx, red[0]);
+    const float mxl = mx * 1.4426950408889634f;
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        int v = tid + i * CLS_BLOCK;
-        if (v < nvalid) {
+        const int v = tid + i * CLS_BLOCK;
+        if (v < nfull) {
 #pragma unroll
-            for (int k = 0; k < VN; k++)
-                if (v * VN + k < V) sum += cls_exp(to_f32(r[i][k]) - mx);
+            for (int k = 0; k < VN; k++) sum += cls_exp_rel(to_f32(r[i][k]), mx, mxl);
         }
     }
+    if (edge) {
+#pragma unroll
+        for (int k = 0; k < VN; k++)
+            if (k < rem) sum += cls_exp_rel(to_f32(re[k]), mx, mxl);
+    }
     sum = block_reduce<false>(sum, red[1]);
-    const float inv = 1.0f / sum;
+    const float inv = 1.0f / sum, inv_dloss = inv * dloss;
 
+    // the vector `w` holds the target column: the loss term
+    auto target_logit = [&](const vecX& w) {
+        float lt = 0.f;
+#pragma unroll
+        for (int k = 0; k < VN; k++)
+            if (k == tk) lt = to_f32(w[k]);               // compare-select: a run-time index would push the row out of registers
+        // -log softmax[target] = (max - logit) + log(sum); accumulates like the reference (fused_classifier.cuh:81)
+        losses[row] += (mx - lt) + logf(sum);
+        return lt;
+    };
+    auto patch_target = [&](vecX& w, float lt) {          // ... and, after the vector's other columns, its gradient
+        const floatX g = from_f32<floatX>((cls_exp_rel(lt, mx, mxl) * inv - 1.0f) * dloss);
+#pragma unroll
+        for (int k = 0; k < VN; k++)
+            if (k == tk) w[k] = g;
+    };
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        int v = tid + i * CLS_BLOCK;
-        if (v < nvalid) {
-            bool has_target = (target / VN) == v;
-            if (has_target) {
-                // -log softmax[target] = (max - logit) + log(sum); accumulates like the reference (:81).
-                // Compare-select instead of r[i][target % VN]: a run-time index would push the row out of registers.
-                float lt = 0.f;
-#pragma unroll
-                for (int k = 0; k < VN; k++)
-                    if (k == target % VN) lt = to_f32(r[i][k]);
-                losses[row] += (mx - lt) + logf(sum);
-            }
+        const int v = tid + i * CLS_BLOCK;
+        if (v < nfull) {
+            float lt = 0.f;
+            const bool has_target = tvec == v;
+            if (has_target) lt = target_logit(r[i]);
             if (WRITE) {
 #pragma unroll
-                for (int k = 0; k < VN; k++) {
-                    int e = v * VN + k;
-                    if (e < V) {
-                        float p = cls_exp(to_f32(r[i][k]) - mx) * inv;
-                        r[i][k] = from_f32<floatX>((p - (e == target ? 1.0f : 0.0f)) * dloss);
-                    }
-                }
+                for (int k = 0; k < VN; k++)
+                    r[i][k] = from_f32<floatX>(cls_scaled(cls_exp_rel(to_f32(r[i][k]), mx, mxl), inv, dloss, inv_dloss));
+                if (has_target) patch_target(r[i], lt);
                 st_vec_nt(x + (size_t)v * VN, r[i]);
             }
+        }
+    }
+    if (edge) {
+        float lt = 0.f;
+        const bool has_target = tvec == nfull;
+        if (has_target) lt = target_logit(re);
+        if (WRITE) {
+#pragma unroll
+            for (int k = 0; k < VN; k++)
+                if (k < rem) re[k] = from_f32<floatX>(cls_scaled(cls_exp_rel(to_f32(re[k]), mx, mxl), inv, dloss, inv_dloss));
+            if (has_target) patch_target(re, lt);
+            st_vec_nt(x + (size_t)nfull * VN, re);       // its padding columns go back as they came
         }
     }
 }
@@ -125,7 +166,7 @@ extern "C" void llmk_fused_classifier(void* logits, float* losses, float dloss, 
     hipStream_t st = (hipStream_t)stream;
     floatX* lg = (floatX*)logits;
     const bool vec_ok = (P % VN == 0) && ((uintptr_t)logits % 16 == 0);
-    const int nvalid = CEIL_DIV(V, VN);
+    const int nvalid = V / VN;                            // full vectors; the straddling one sits beside them
     llmk::ProfScope prof("fused_classifier", 0, (write_dlogits ? 2.0 : 1.0) * N * (double)P * sizeof(floatX), st);
 #define CLS_LAUNCH(NVT)                                                                                     \
     do {                                                                                                    \
