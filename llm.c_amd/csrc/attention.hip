@@ -717,12 +717,10 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
                 pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
             }
-            f32x4 d4[4];
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int rr = 32 * qb + g * 8 + half * 4;
                 const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
-                d4[g] = fa_lds_f32x4(stat_d + rr * 4);
 #pragma unroll
                 for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
             }
@@ -734,9 +732,11 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 }
             }
 #pragma unroll
-            for (int g = 0; g < 4; g++)
+            for (int g = 0; g < 4; g++) {
+                const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);     // rowsum(dO*O) of the four queries, read where it is used
 #pragma unroll
-                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[g][e]);
+                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[e]);
+            }
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
                 const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
