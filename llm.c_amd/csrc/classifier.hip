@@ -29,6 +29,24 @@ __device__ __forceinline__ float cls_exp_rel(float x, float, float mxl) { return
 __device__ __forceinline__ float cls_scaled(float e, float, float, float inv_dloss) { return e * inv_dloss; }
 #endif
 
+// The row's vectors are addressed through a buffer descriptor: one per-lane byte offset (16 * lane) plus a scalar
+// offset per vector slot. With plain pointers the compiler keeps one per-lane offset per slot alive from the loads to
+// the stores; seven of them do not fit beside the row in 64 registers and went to scratch memory and back, a quarter
+// more traffic than the logits themselves.
+typedef int cls_i4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t cls_row_rsrc(floatX* row, int bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(row, 0, bytes, 0x00020000);   // raw buffer, 32-bit data format
+}
+__device__ __forceinline__ vecX cls_ld(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int slot_bytes) {
+    const cls_i4 q = __builtin_amdgcn_raw_buffer_load_b128(rs, lane_bytes, slot_bytes, 0);
+    vecX out;
+    *reinterpret_cast<cls_i4*>(&out) = q;
+    return out;
+}
+__device__ __forceinline__ void cls_st_nt(__amdgpu_buffer_rsrc_t rs, int lane_bytes, int slot_bytes, const vecX& w) {
+    __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const cls_i4*>(&w), rs, lane_bytes, slot_bytes, 2 /* nt */);
+}
+
 // NVT: 16-byte vectors held per lane; requires P/VN <= NVT*CLS_BLOCK.
 // The vectors whose VN columns are all real ([0, V/VN)) take loops without any per-element test; the one vector
 // that straddles V (when V is not a multiple of VN) is held by a single lane and handled on the side, and the
@@ -47,15 +65,40 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     const int tvec = target / VN, tk = target - tvec * VN;
     const bool edge = rem != 0 && tid == nfull % CLS_BLOCK;   // this lane holds the straddling vector
 
+    const __amdgpu_buffer_rsrc_t rs = cls_row_rsrc(x, P * (int)sizeof(floatX));
+    const int lane_bytes = tid * 16;
+
     vecX r[NVT], re;
     float mx = -INFINITY;
+    // The row stays in registers as loaded. Without this the compiler carries converted or unpacked columns from one
+    // pass into the next, which takes more registers than there are and ends in scratch memory.
+    auto keep_packed = [&]() {
+#pragma unroll
+        for (int i = 0; i < NVT; i++) {
+            unsigned* w32 = reinterpret_cast<unsigned*>(&r[i]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) asm volatile("" : "+v"(w32[q]));
+        }
+    };
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
         const int v = tid + i * CLS_BLOCK;
         if (v < nfull) {
-            r[i] = ld_vec(x + (size_t)v * VN);
+            r[i] = cls_ld(rs, lane_bytes, i * CLS_BLOCK * 16);
+            if (WRITE) {
 #pragma unroll
-            for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
+                for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
+            }
+        }
+    }
+    if (!WRITE) {   // no store needs the vectors whole, so they are pinned as loaded before their first use too
+        keep_packed();
+#pragma unroll
+        for (int i = 0; i < NVT; i++) {
+            if (tid + i * CLS_BLOCK < nfull) {
+#pragma unroll
+                for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
+            }
         }
     }
     if (edge) {
@@ -66,6 +109,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     }
     mx = block_reduce<true>(mx, red[0]);
     const float mxl = mx * 1.4426950408889634f;
+    keep_packed();
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
@@ -82,22 +126,37 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     }
     sum = block_reduce<false>(sum, red[1]);
     const float inv = 1.0f / sum, inv_dloss = inv * dloss;
+    keep_packed();
 
-    // the vector `w` holds the target column: the loss term
+    // The vector `w` holds the target column: the loss term. The column is picked as a 32-bit word by compare-select
+    // (a run-time index would push the row out of registers) and, in bf16, as one half of that word: converting all
+    // columns here made the compiler carry the converted values into the exponent loop, through scratch memory.
+    constexpr int PER_WORD = VN / 4;                       // 2 bf16 or 1 fp32 per 32-bit word
+    const int tq = tk / PER_WORD, th = tk - tq * PER_WORD;
     auto target_logit = [&](const vecX& w) {
-        float lt = 0.f;
+        const unsigned* w32 = reinterpret_cast<const unsigned*>(&w);
+        unsigned word = 0;
 #pragma unroll
-        for (int k = 0; k < VN; k++)
-            if (k == tk) lt = to_f32(w[k]);               // compare-select: a run-time index would push the row out of registers
+        for (int q = 0; q < 4; q++)
+            if (q == tq) word = w32[q];
+        const float lt = __uint_as_float(PER_WORD == 1 ? word : th ? word & 0xffff0000u : word << 16);
         // -log softmax[target] = (max - logit) + log(sum); accumulates like the reference (fused_classifier.cuh:81)
         losses[row] += (mx - lt) + logf(sum);
         return lt;
     };
     auto patch_target = [&](vecX& w, float lt) {          // ... and, after the vector's other columns, its gradient
-        const floatX g = from_f32<floatX>((cls_exp_rel(lt, mx, mxl) * inv - 1.0f) * dloss);
+        const float gf = (cls_exp_rel(lt, mx, mxl) * inv - 1.0f) * dloss;
+        unsigned* w32 = reinterpret_cast<unsigned*>(&w);
+        unsigned bits;
+        if constexpr (PER_WORD == 1) {
+            bits = __float_as_uint(gf);
+        } else {
+            const __bf16 g = from_f32<__bf16>(gf);
+            bits = (unsigned)__builtin_bit_cast(unsigned short, g);
+        }
 #pragma unroll
-        for (int k = 0; k < VN; k++)
-            if (k == tk) w[k] = g;
+        for (int q = 0; q < 4; q++)
+            if (q == tq) w32[q] = PER_WORD == 1 ? bits : th ? (w32[q] & 0x0000ffffu) | (bits << 16) : (w32[q] & 0xffff0000u) | bits;
     };
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
@@ -111,7 +170,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
                 for (int k = 0; k < VN; k++)
                     r[i][k] = from_f32<floatX>(cls_scaled(cls_exp_rel(to_f32(r[i][k]), mx, mxl), inv, dloss, inv_dloss));
                 if (has_target) patch_target(r[i], lt);
-                st_vec_nt(x + (size_t)v * VN, r[i]);
+                cls_st_nt(rs, lane_bytes, i * CLS_BLOCK * 16, r[i]);
             }
         }
     }
