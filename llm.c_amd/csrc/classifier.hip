@@ -47,13 +47,15 @@ __device__ __forceinline__ void cls_st_nt(__amdgpu_buffer_rsrc_t rs, int lane_by
     __builtin_amdgcn_raw_buffer_store_b128(*reinterpret_cast<const cls_i4*>(&w), rs, lane_bytes, slot_bytes, 2 /* nt */);
 }
 
-// NVT: 16-byte vectors held per lane; requires P/VN <= NVT*CLS_BLOCK.
+// NVT: 16-byte vectors held per lane of a BLK-lane workgroup; requires V/VN <= NVT*BLK. A CU holds 2048 lanes: two
+// rows with 1024-lane workgroups, three with 512-lane ones when the row fits their registers (13 vectors, 70 registers,
+// six waves per SIMD), which measured 4 % faster on GPT-2's vocabulary.
 // The vectors whose VN columns are all real ([0, V/VN)) take loops without any per-element test; the one vector
 // that straddles V (when V is not a multiple of VN) is held by a single lane and handled on the side, and the
 // target column is patched in the one vector that holds it. Per element that leaves: max; fma, exp2, add; and
 // fma, exp2, multiply, convert.
-template <int NVT, bool WRITE>
-__global__ void __launch_bounds__(CLS_BLOCK, NVT <= 7 ? 8 : 4)   // up to 7 vectors: 64 registers, two workgroups (rows) per CU
+template <int NVT, bool WRITE, int BLK = CLS_BLOCK>
+__global__ void __launch_bounds__(BLK, BLK == 512 ? 6 : NVT <= 7 ? 8 : 4)
 fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses, float dloss,
                         const int* __restrict__ targets, int V, int P) {
     __shared__ float red[2][16];
@@ -63,7 +65,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     const int tid = threadIdx.x;
     const int target = targets[row];
     const int tvec = target / VN, tk = target - tvec * VN;
-    const bool edge = rem != 0 && tid == nfull % CLS_BLOCK;   // this lane holds the straddling vector
+    const bool edge = rem != 0 && tid == nfull % BLK;   // this lane holds the straddling vector
 
     const __amdgpu_buffer_rsrc_t rs = cls_row_rsrc(x, P * (int)sizeof(floatX));
     const int lane_bytes = tid * 16;
@@ -82,9 +84,9 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     };
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        const int v = tid + i * CLS_BLOCK;
+        const int v = tid + i * BLK;
         if (v < nfull) {
-            r[i] = cls_ld(rs, lane_bytes, i * CLS_BLOCK * 16);
+            r[i] = cls_ld(rs, lane_bytes, i * BLK * 16);
             if (WRITE) {
 #pragma unroll
                 for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
@@ -95,7 +97,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
         keep_packed();
 #pragma unroll
         for (int i = 0; i < NVT; i++) {
-            if (tid + i * CLS_BLOCK < nfull) {
+            if (tid + i * BLK < nfull) {
 #pragma unroll
                 for (int k = 0; k < VN; k++) mx = fmaxf(mx, to_f32(r[i][k]));
             }
@@ -113,7 +115,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     float sum = 0.f;
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        const int v = tid + i * CLS_BLOCK;
+        const int v = tid + i * BLK;
         if (v < nfull) {
 #pragma unroll
             for (int k = 0; k < VN; k++) sum += cls_exp_rel(to_f32(r[i][k]), mx, mxl);
@@ -160,7 +162,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
     };
 #pragma unroll
     for (int i = 0; i < NVT; i++) {
-        const int v = tid + i * CLS_BLOCK;
+        const int v = tid + i * BLK;
         if (v < nfull) {
             float lt = 0.f;
             const bool has_target = tvec == v;
@@ -170,7 +172,7 @@ fused_classifier_kernel(floatX* __restrict__ logits, float* __restrict__ losses,
                 for (int k = 0; k < VN; k++)
                     r[i][k] = from_f32<floatX>(cls_scaled(cls_exp_rel(to_f32(r[i][k]), mx, mxl), inv, dloss, inv_dloss));
                 if (has_target) patch_target(r[i], lt);
-                cls_st_nt(rs, lane_bytes, i * CLS_BLOCK * 16, r[i]);
+                cls_st_nt(rs, lane_bytes, i * BLK * 16, r[i]);
             }
         }
     }
@@ -227,15 +229,17 @@ extern "C" void llmk_fused_classifier(void* logits, float* losses, float dloss, 
     const bool vec_ok = (P % VN == 0) && ((uintptr_t)logits % 16 == 0);
     const int nvalid = V / VN;                            // full vectors; the straddling one sits beside them
     llmk::ProfScope prof("fused_classifier", 0, (write_dlogits ? 2.0 : 1.0) * N * (double)P * sizeof(floatX), st);
-#define CLS_LAUNCH(NVT)                                                                                     \
+#define CLS_LAUNCH(NVT, BLK)                                                                                \
     do {                                                                                                    \
-        if (write_dlogits) fused_classifier_kernel<NVT, true><<<N, CLS_BLOCK, 0, st>>>(lg, losses, dloss, targets, V, P); \
-        else fused_classifier_kernel<NVT, false><<<N, CLS_BLOCK, 0, st>>>(lg, losses, dloss, targets, V, P);            \
+        if (write_dlogits) fused_classifier_kernel<NVT, true, BLK><<<N, BLK, 0, st>>>(lg, losses, dloss, targets, V, P); \
+        else fused_classifier_kernel<NVT, false, BLK><<<N, BLK, 0, st>>>(lg, losses, dloss, targets, V, P);            \
     } while (0)
-    if (vec_ok && nvalid <= 2 * CLS_BLOCK) CLS_LAUNCH(2);
-    else if (vec_ok && nvalid <= 4 * CLS_BLOCK) CLS_LAUNCH(4);
-    else if (vec_ok && nvalid <= 7 * CLS_BLOCK) CLS_LAUNCH(7);
-    else if (vec_ok && nvalid <= 13 * CLS_BLOCK) CLS_LAUNCH(13);
+    if (vec_ok && nvalid <= 2 * CLS_BLOCK) CLS_LAUNCH(2, CLS_BLOCK);
+    else if (vec_ok && nvalid <= 4 * CLS_BLOCK) CLS_LAUNCH(4, CLS_BLOCK);
+    else if (vec_ok && nvalid <= 13 * 512 && write_dlogits)       // GPT-2's vocabulary in bf16: three rows per CU at 70 registers
+        fused_classifier_kernel<13, true, 512><<<N, 512, 0, st>>>(lg, losses, dloss, targets, V, P);
+    else if (vec_ok && nvalid <= 7 * CLS_BLOCK) CLS_LAUNCH(7, CLS_BLOCK);
+    else if (vec_ok && nvalid <= 13 * CLS_BLOCK) CLS_LAUNCH(13, CLS_BLOCK);
     else {
         if (write_dlogits) fused_classifier_generic_kernel<true><<<N, CLS_BLOCK, 0, st>>>(lg, losses, dloss, targets, V, P);
         else fused_classifier_generic_kernel<false><<<N, CLS_BLOCK, 0, st>>>(lg, losses, dloss, targets, V, P);

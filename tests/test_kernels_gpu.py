@@ -217,7 +217,8 @@ def test_gelu_backward_bias_equals_the_two_separate_steps(precision, N, OC):
 
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("precision", PRECS)
-@pytest.mark.parametrize("N,V,P", [(5, 100, 128), (64, 50257, 50304), (3, 8003, 8064), (2, 130000, 130048)])
+@pytest.mark.parametrize("N,V,P", [(5, 100, 128), (64, 50257, 50304), (3, 8003, 8064), (2, 130000, 130048),
+                                   (3, 20000, 20032), (2, 55003, 55040), (2, 28001, 28032)])   # one shape per kernel variant
 def test_fused_classifier(precision, N, V, P):
     L = G.lib(precision)
     z = rnd((N, P), 0, 2.0)
