@@ -42,6 +42,10 @@ void gpt2_allocate_state(LLMK_GPT2* m, int B, int T);
 void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T);
 /* gpt2_validate, train_gpt2.cu:761. Returns the mean loss; per-token losses via gpt2_cpu_losses. */
 float gpt2_validate(LLMK_GPT2* m, const int* inputs, const int* targets, size_t B, size_t T);
+/* The text-generation loop of the reference's main, train_gpt2.cu:1751-1796 (minus the printing). gen_tokens: host,
+ * batch*seq_len ints as allocated; on return positions 1..genT-1 of the first sequence hold the sampled tokens and
+ * everything else eot_token. sample_rng_state: llmc/sampler.h's xorshift state (the reference restarts it at 1337). */
+void gpt2_generate(LLMK_GPT2* m, int* gen_tokens, int genT, int eot_token, unsigned long long* sample_rng_state);
 /* gpt2_backward_and_reduce, train_gpt2.cu:788 (the reduce is a no-op on one GPU) */
 void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* targets, int grad_accum_steps, int micro_step);
 /* gpt2_calculate_grad_norm, train_gpt2.cu:992 */

@@ -79,6 +79,7 @@ DRIVER_ABI = {
     "gpt2_allocate_state": (None, [vp, i32, i32]),
     "gpt2_forward": (None, [vp, vp, sz, sz]),
     "gpt2_validate": (f32, [vp, vp, vp, sz, sz]),
+    "gpt2_generate": (None, [vp, vp, i32, i32, C.POINTER(C.c_ulonglong)]),
     "gpt2_backward_and_reduce": (None, [vp, vp, vp, i32, i32]),
     "gpt2_calculate_grad_norm": (f32, [vp]),
     "gpt2_update": (None, [vp, f32, f32, f32, f32, f32, f32, i32, i32]),

@@ -465,6 +465,28 @@ float gpt2_validate(LLMK_GPT2* m, const int* inputs, const int* targets, size_t 
     return mean_loss / (float)(B * T);
 }
 
+// The generation loop of the reference's trainer (train_gpt2.cu:1751-1796), without the printing: every position of
+// gen_tokens starts as eot_token, then positions 1..genT-1 are drawn one at a time from the model's distribution after
+// the tokens before them. Each draw runs the forward pass on one sequence whose length is rounded up to a multiple of
+// min(seq_len, 256) (no KV cache, as there), moves the logits of the last real position to the host and samples there
+// with llmc/sampler.h's generator, whose state the caller owns (the reference starts it at 1337 for every generation).
+void gpt2_generate(LLMK_GPT2* m, int* gen_tokens, int genT, int eot_token, unsigned long long* sample_rng_state) {
+    const int B = m->batch_size, T = m->seq_len, V = m->config.vocab_size;
+    const size_t Vp = m->config.padded_vocab_size;
+    if (genT > T) { printf("gpt2_generate: genT=%d exceeds the sequence length %d\n", genT, T); exit(EXIT_FAILURE); }
+    for (int i = 0; i < B * T; i++) gen_tokens[i] = eot_token;
+    std::vector<char> raw((size_t)V * m->X);
+    std::vector<float> cpu_logits(V);
+    const int chunk = T < 256 ? T : 256;
+    for (int t = 1; t < genT; t++) {
+        gpt2_forward(m, gen_tokens, 1, (size_t)((t + chunk - 1) / chunk) * chunk);
+        hipCheck(hipMemcpy(raw.data(), off(m->acts.output, (size_t)(t - 1) * Vp, m->X), (size_t)V * m->X, hipMemcpyDeviceToHost));
+        from_storage(cpu_logits.data(), raw.data(), V, m->X);
+        const float coin = llmk::random_f32(sample_rng_state);
+        gen_tokens[t] = llmk::sample_softmax(cpu_logits.data(), V, coin);
+    }
+}
+
 void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* targets, int grad_accum_steps, int micro_step) {
     if (m->grads_memory == nullptr) { fprintf(stderr, "Need to allocate gradients before backward"); exit(EXIT_FAILURE); }
     const bool last_step = micro_step == grad_accum_steps - 1;

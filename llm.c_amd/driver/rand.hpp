@@ -85,4 +85,21 @@ inline uint32_t random_u32(unsigned long long* state) {
     return (uint32_t)((*state * 0x2545F4914F6CDD1Dull) >> 32);
 }
 
+// random float32 in [0,1) from the same stream (reference: llmc/sampler.h:18-20)
+inline float random_f32(unsigned long long* state) { return (random_u32(state) >> 8) / 16777216.0f; }
+
+// Index drawn from softmax(logits) with the uniform number `coin` (reference: llmc/sampler.h:22-40): the
+// normaliser is summed in double, the running distribution in float, and the coin is scaled instead of the terms.
+inline int sample_softmax(const float* logits, int n, float coin) {
+    double norm = 0;
+    for (int i = 0; i < n; i++) norm += expf(logits[i]);
+    coin *= norm;
+    float cdf = 0.0f;
+    for (int i = 0; i < n; i++) {
+        cdf += expf(logits[i]);
+        if (coin < cdf) return i;
+    }
+    return n - 1;
+}
+
 }  // namespace llmk

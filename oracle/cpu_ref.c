@@ -716,6 +716,77 @@ CREF_API int cref_gpt2_train(const cref_config* cfg, float* params, const int* i
     return 0;
 }
 
+/* ------------------------------------------------------------------------------------------
+ * Text generation: forward only + the sampler (train_gpt2.cu:1751-1796, llmc/sampler.h)
+ * ---------------------------------------------------------------------------------------- */
+
+/* random float32 in [0,1) (llmc/sampler.h:18-20) */
+CREF_API float cref_random_f32(uint64_t* state) { return (cref_random_u32(state) >> 8) / 16777216.0f; }
+
+/* index drawn from softmax(logits) with the uniform number coin (llmc/sampler.h:22-40) */
+CREF_API int cref_sample_softmax(const float* logits, int n, float coin) {
+    double norm = 0;
+    for (int i = 0; i < n; i++) norm += expf(logits[i]);
+    coin *= norm;
+    float cdf = 0.0f;
+    for (int i = 0; i < n; i++) {
+        cdf += expf(logits[i]);
+        if (coin < cdf) return i;
+    }
+    return n - 1;
+}
+
+/* logits[B*T*Vp] of the forward pass alone (same order of operations as cref_gpt2_train's forward half,
+ * train_gpt2.c:765-880); one layer's activations are kept at a time */
+CREF_API int cref_gpt2_logits(const cref_config* cfg, const float* params, const int* inputs, int B, int T, float* logits) {
+    const int C = cfg->channels, L = cfg->num_layers, NH = cfg->num_heads, Vp = cfg->padded_vocab_size;
+    const size_t N = (size_t)B * T;
+    size_t sz[CREF_NPARAM];
+    const float* P[CREF_NPARAM];
+    cref_param_sizes(sz, cfg);
+    { size_t o = 0; for (int i = 0; i < CREF_NPARAM; i++) { P[i] = params + o; o += sz[i]; } }
+    float* res = falloc(N * C); float* res2 = falloc(N * C); float* ln = falloc(N * C); float* tmp_c = falloc(N * C);
+    float* mean = falloc(N); float* rstd = falloc(N);
+    float* qkv = falloc(N * 3 * C); float* atty = falloc(N * C); float* att = falloc((size_t)B * NH * T * T);
+    float* fch = falloc(N * 4 * C); float* fch_gelu = falloc(N * 4 * C);
+    cref_encoder_forward(res, inputs, P[0], P[1], B, T, C);
+    for (int l = 0; l < L; l++) {
+        cref_layernorm_forward(ln, mean, rstd, res, P[2] + (size_t)l * C, P[3] + (size_t)l * C, (int)N, C);
+        cref_matmul_forward(qkv, ln, P[4] + (size_t)l * 3 * C * C, P[5] + (size_t)l * 3 * C, (int)N, C, 3 * C);
+        cref_attention_forward(atty, att, NULL, qkv, B, T, C, NH);
+        cref_matmul_forward(tmp_c, atty, P[6] + (size_t)l * C * C, P[7] + (size_t)l * C, (int)N, C, C);
+        cref_residual_forward(res2, res, tmp_c, N * C);
+        cref_layernorm_forward(ln, mean, rstd, res2, P[8] + (size_t)l * C, P[9] + (size_t)l * C, (int)N, C);
+        cref_matmul_forward(fch, ln, P[10] + (size_t)l * 4 * C * C, P[11] + (size_t)l * 4 * C, (int)N, C, 4 * C);
+        cref_gelu_forward(fch_gelu, fch, N * 4 * C);
+        cref_matmul_forward(tmp_c, fch_gelu, P[12] + (size_t)l * 4 * C * C, P[13] + (size_t)l * C, (int)N, 4 * C, C);
+        cref_residual_forward(res, res2, tmp_c, N * C);
+    }
+    cref_layernorm_forward(ln, mean, rstd, res, P[14], P[15], (int)N, C);
+    cref_matmul_forward(logits, ln, P[0], NULL, (int)N, C, Vp);
+    free(res); free(res2); free(ln); free(tmp_c); free(mean); free(rstd); free(qkv); free(atty); free(att);
+    free(fch); free(fch_gelu);
+    return 0;
+}
+
+/* The generation loop of train_gpt2.cu:1751-1796: tokens[0..T) start as eot_token; position t = 1..genT-1 is sampled
+ * from the logits at position t-1 of a forward pass over one sequence of length ceil(t / min(T,256)) * min(T,256). */
+CREF_API int cref_gpt2_generate(const cref_config* cfg, const float* params, int* tokens, int T, int genT, int eot_token,
+                                uint64_t* rng_state) {
+    const int V = cfg->vocab_size, Vp = cfg->padded_vocab_size;
+    const int chunk = T < 256 ? T : 256;
+    float* logits = falloc((size_t)T * Vp);
+    for (int i = 0; i < T; i++) tokens[i] = eot_token;
+    for (int t = 1; t < genT; t++) {
+        const int Tr = (t + chunk - 1) / chunk * chunk;
+        cref_gpt2_logits(cfg, params, tokens, 1, Tr, logits);
+        const float coin = cref_random_f32(rng_state);
+        tokens[t] = cref_sample_softmax(logits + (size_t)(t - 1) * Vp, V, coin);
+    }
+    free(logits);
+    return 0;
+}
+
 CREF_API int cref_num_threads(void) {
 #ifdef _OPENMP
     return omp_get_max_threads();

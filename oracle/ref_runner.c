@@ -11,6 +11,9 @@
  */
 #define TESTING
 #include "train_gpt2.c"
+/* the sampler of the reference's GPU trainer (random_u32, random_f32, sample_softmax): a plain C header. The CPU
+ * trainer's own copies of the first two sit behind #ifndef TESTING (train_gpt2.c:1046-1073), so nothing clashes. */
+#include "llmc/sampler.h"
 
 /* Runs the reference's own gpt2_forward / gpt2_zero_grad / gpt2_backward / gpt2_update
  * (train_gpt2.c:1163-1169 call order) for `steps` steps on one fixed batch.
@@ -34,6 +37,24 @@ int ref_gpt2_train(const char* ckpt, int* inputs, int* targets, int B, int T, in
         if (step_ms_out) step_ms_out[s] = (float)((t1.tv_sec - t0.tv_sec) * 1e3 + (t1.tv_nsec - t0.tv_nsec) * 1e-6);
     }
     if (params_out) memcpy(params_out, model.params_memory, model.num_parameters * sizeof(float));
+    gpt2_free(&model);
+    return 0;
+}
+
+/* The generation loop of train_gpt2.cu:1751-1796 put together from the reference's own parts: its CPU forward pass
+ * (train_gpt2.c gpt2_forward, on one sequence of the rounded length) and llmc/sampler.h. */
+int ref_gpt2_generate(const char* ckpt, int* tokens, int T, int genT, int eot_token, unsigned long long* rng_state) {
+    GPT2 model;
+    gpt2_build_from_checkpoint(&model, ckpt);
+    const int V = model.config.vocab_size, Vp = model.config.padded_vocab_size;
+    const int chunk = T < 256 ? T : 256;
+    for (int i = 0; i < T; i++) tokens[i] = eot_token;
+    gpt2_forward(&model, tokens, NULL, 1, (size_t)T);     /* sizes the activations for the longest sequence */
+    for (int t = 1; t < genT; t++) {
+        gpt2_forward(&model, tokens, NULL, 1, (size_t)((t + chunk - 1) / chunk * chunk));
+        float coin = random_f32(rng_state);
+        tokens[t] = sample_softmax(model.acts.logits + (size_t)(t - 1) * Vp, V, coin);
+    }
     gpt2_free(&model);
     return 0;
 }

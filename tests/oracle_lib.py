@@ -88,6 +88,14 @@ def cref():
                                   C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, C.c_float, C.c_int,
                                   f32p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     L.cref_gpt2_train.restype = C.c_int
+    L.cref_random_f32.argtypes = [C.POINTER(C.c_uint64)]
+    L.cref_random_f32.restype = C.c_float
+    L.cref_sample_softmax.argtypes = [f32p, C.c_int, C.c_float]
+    L.cref_sample_softmax.restype = C.c_int
+    L.cref_gpt2_logits.argtypes = [C.POINTER(Config), f32p, i32p, C.c_int, C.c_int, f32p]
+    L.cref_gpt2_logits.restype = C.c_int
+    L.cref_gpt2_generate.argtypes = [C.POINTER(Config), f32p, i32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_uint64)]
+    L.cref_gpt2_generate.restype = C.c_int
     L.cref_num_threads.restype = C.c_int
     _cref = L
     return L
@@ -123,6 +131,12 @@ def ref():
                                  C.c_float, C.c_float, C.c_float, C.c_float, C.c_float,
                                  f32p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
     L.ref_gpt2_train.restype = C.c_int
+    L.random_f32.argtypes = [C.POINTER(C.c_uint64)]
+    L.random_f32.restype = C.c_float
+    L.sample_softmax.argtypes = [f32p, C.c_int, C.c_float]
+    L.sample_softmax.restype = C.c_int
+    L.ref_gpt2_generate.argtypes = [C.c_char_p, i32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_uint64)]
+    L.ref_gpt2_generate.restype = C.c_int
     L.ref_num_threads.restype = C.c_int
     _ref = L
     return L
@@ -180,6 +194,22 @@ def ref_train(ckpt_path, cfg, inputs, targets, B, T, steps, lr=1e-4, b1=0.9, b2=
                               losses, _opt(grads), grad_step, _opt(logits), _opt(ms), _opt(pout))
     assert rc == 0
     return dict(losses=losses, grads=grads, logits=logits, step_ms=ms, params=pout)
+
+
+def cref_generate(cfg, params, T, genT, eot_token, rng_seed=1337):
+    """Tokens of the CPU restatement's generation loop (positions >= genT stay eot_token)."""
+    tokens = np.zeros(T, dtype=np.int32)
+    state = C.c_uint64(rng_seed)
+    assert cref().cref_gpt2_generate(C.byref(cfg), params, tokens, T, genT, eot_token, C.byref(state)) == 0
+    return tokens, state.value
+
+
+def ref_generate(ckpt_path, T, genT, eot_token, rng_seed=1337):
+    """The same loop run by the compiled reference (its CPU forward pass + llmc/sampler.h)."""
+    tokens = np.zeros(T, dtype=np.int32)
+    state = C.c_uint64(rng_seed)
+    assert ref().ref_gpt2_generate(ckpt_path.encode(), tokens, T, genT, eot_token, C.byref(state)) == 0
+    return tokens, state.value
 
 
 def to_bf16_bits(x):

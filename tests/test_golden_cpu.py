@@ -37,3 +37,12 @@ def test_oracle_reproduces_reference_fixture():
     r3 = ol.cref_train(cfg, params, g["inputs"], g["targets"], B, T, 4, lr=lr, b1=b1, b2=b2, eps=eps, wd=wd, grad_step=3)
     scale3 = np.abs(g["grad_val_step3"]).max()
     assert np.abs(r3["grads"][g["grad_idx"]] - g["grad_val_step3"]).max() <= 2e-4 * scale3
+
+
+def test_oracle_reproduces_reference_generation_fixture():
+    g = np.load(os.path.join(os.path.dirname(GOLD), "tiny_gpt2_generate.npz"))
+    cfg = ol.Config(*[int(x) for x in g["config"]])
+    params = np.ascontiguousarray(ol.init_params(cfg, int(g["seed"])) * np.float32(g["param_scale"]), np.float32)
+    tokens, state = ol.cref_generate(cfg, params, cfg.max_seq_len, int(g["genT"]), int(g["eot_token"]), int(g["rng_seed"]))
+    np.testing.assert_array_equal(tokens, g["tokens"])
+    assert state == int(g["rng_state_after"])

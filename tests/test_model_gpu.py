@@ -272,6 +272,51 @@ def test_validate_matches_training_forward_loss():
     m.free()
 
 
+def test_fp32_generation_matches_reference_fixture():
+    """The reference's sampling loop (train_gpt2.cu:1751-1796) through the driver: token for token what the
+    reference's CPU forward pass and llmc/sampler.h produced (tests/golden/tiny_gpt2_generate.npz)."""
+    g = np.load(os.path.join(os.path.dirname(GOLD), "tiny_gpt2_generate.npz"))
+    cfg = ol.Config(*[int(x) for x in g["config"]])
+    params = np.ascontiguousarray(ol.init_params(cfg, int(g["seed"])) * np.float32(g["param_scale"]), np.float32)
+    B, T = 2, cfg.max_seq_len
+    m = Model("fp32", cfg, B, T, params=params, master=0)
+    tokens = np.zeros(B * T, np.int32)
+    state = C.c_ulonglong(int(g["rng_seed"]))
+    m.L.gpt2_generate(m.h, tokens.ctypes.data_as(C.c_void_p), int(g["genT"]), int(g["eot_token"]), C.byref(state))
+    np.testing.assert_array_equal(tokens[:T], g["tokens"])
+    assert (tokens[T:] == int(g["eot_token"])).all()
+    assert state.value == int(g["rng_state_after"])
+    m.free()
+
+
+def test_bf16_generation_samples_from_its_own_logits():
+    """bf16 logits differ from the CPU's, so the tokens may too; what must hold is that each token is the sampler's
+    answer for the logits the model produced on the tokens before it, also when the rounded sequence length changes
+    (256 -> 512 at position 257)."""
+    cfg = ol.Config(512, 300, 320, 2, 2, 128)
+    B, T, genT, eot = 1, 512, 260, 299
+    params = np.ascontiguousarray(ol.init_params(cfg, 11) * np.float32(8), np.float32)
+    m = Model("bf16", cfg, B, T, params=params)
+    tokens = np.zeros(B * T, np.int32)
+    state = C.c_ulonglong(1337)
+    m.L.gpt2_generate(m.h, tokens.ctypes.data_as(C.c_void_p), genT, eot, C.byref(state))
+    assert ((tokens >= 0) & (tokens < cfg.vocab_size)).all() and (tokens[genT:] == eot).all() and tokens[0] == eot
+    assert len(set(tokens[1:genT].tolist())) > 20
+    # causal model: one forward pass over the finished sequence gives every position's logits again
+    m.L.gpt2_forward(m.h, tokens.ctypes.data_as(C.c_void_p), 1, T)
+    lg = m.logits(cfg.padded_vocab_size).reshape(T, cfg.padded_vocab_size)
+    st = C.c_uint64(1337)
+    agree = 0
+    for t in range(1, genT):
+        coin = ol.cref().cref_random_f32(C.byref(st))
+        agree += ol.cref().cref_sample_softmax(np.ascontiguousarray(lg[t - 1, :cfg.vocab_size]), cfg.vocab_size, coin) == tokens[t]
+    # the same position computed inside a sequence of another length can round differently in bf16; a coin has to land
+    # within that rounding of a boundary of the distribution for the token to change
+    assert agree >= genT - 1 - 3, agree
+    assert st.value == state.value
+    m.free()
+
+
 def test_bf16_full_size_step_properties():
     """B=64, T=1024, 124M: the shape the throughput is quoted on. The oracle cannot run it, so check
     what must hold at any size: initial loss ~ ln(V), loss decreases on a repeated batch, finite gradient norm,

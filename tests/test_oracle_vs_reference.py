@@ -275,6 +275,59 @@ def test_whole_model_matches_compiled_reference():
     np.testing.assert_allclose(c["params"], r["params"], rtol=1e-4, atol=1e-4)
 
 
+def test_sampler_closed_forms():
+    L = ol.cref()
+    # four equally likely outcomes: the coin's quarter picks the index
+    u = np.zeros(4, np.float32)
+    assert [L.cref_sample_softmax(u, 4, c) for c in (0.0, 0.3, 0.5, 0.76, 0.999)] == [0, 1, 2, 3, 3]
+    # one outcome far more likely than the rest takes (almost) every coin; softmax is shift-invariant
+    z = np.array([0.0, 40.0, 0.0], np.float32)
+    assert all(L.cref_sample_softmax(z, 3, c) == 1 for c in (1e-6, 0.5, 0.999999))
+    assert L.cref_sample_softmax(z, 3, 0.0) == 0
+    z = np.array([1.0, 2.0, 3.0, 0.5], np.float32)
+    p = np.exp(z.astype(np.float64)); cdf = np.cumsum(p / p.sum())
+    for c in (0.05, 0.2, 0.5, 0.9, 0.99):
+        assert L.cref_sample_softmax(z, 4, c) == int(np.searchsorted(cdf, c, side="right"))
+    # the generator: floats with 24 random bits in [0, 1), from the documented xorshift* recurrence
+    st = C.c_uint64(1337)
+    x = 1337
+    for _ in range(5):
+        x ^= x >> 12; x ^= (x << 25) & (2**64 - 1); x ^= x >> 27
+        want = ((((x * 0x2545F4914F6CDD1D) & (2**64 - 1)) >> 32) >> 8) / 16777216.0
+        assert L.cref_random_f32(C.byref(st)) == np.float32(want)
+        assert st.value == x
+
+
+@needs_ref
+def test_sampler_matches_compiled_reference():
+    L, R = ol.cref(), ol.ref()
+    for seed in (1337, 1, 0xDEADBEEFCAFE):
+        a, b = C.c_uint64(seed), C.c_uint64(seed)
+        for _ in range(64):
+            assert L.cref_random_f32(C.byref(a)) == R.random_f32(C.byref(b))
+        assert a.value == b.value
+    rs = np.random.RandomState(3)
+    for n in (7, 100, 50257):
+        z = (rs.randn(n) * 3).astype(np.float32)
+        for coin in [0.0, 0.999999] + list(rs.rand(40).astype(np.float32)):
+            assert L.cref_sample_softmax(z, n, coin) == R.sample_softmax(z, n, coin)
+
+
+@needs_ref
+def test_generation_matches_compiled_reference():
+    cfg = Config(**TINY)
+    params = ol.init_params(cfg, 42) * 8      # sharper distributions than the 0.02-scale init gives
+    params = np.ascontiguousarray(params, np.float32)
+    with tempfile.TemporaryDirectory() as d:
+        path = os.path.join(d, "tiny.bin")
+        assert ol.cref().cref_write_checkpoint_fp32(path.encode(), params, C.byref(cfg)) == 0
+        rt, rstate = ol.ref_generate(path, cfg.max_seq_len, 32, cfg.vocab_size - 1)
+    ct, cstate = ol.cref_generate(cfg, params, cfg.max_seq_len, 32, cfg.vocab_size - 1)
+    np.testing.assert_array_equal(ct, rt)
+    assert cstate == rstate
+    assert len(set(ct[1:].tolist())) > 8      # a sequence, not one token over and over
+
+
 def test_whole_model_gradient_by_finite_differences():
     # brute force: central differences of the oracle's own loss on a few coordinates of every tensor
     cfg = Config(max_seq_len=8, vocab_size=20, padded_vocab_size=32, num_layers=1, num_heads=2, channels=16)
