@@ -62,6 +62,11 @@ void gpt2_free(LLMK_GPT2* m);
  * ignored: the data loader is outside this library). load_state needs gpt2_allocate_state first. */
 void gpt2_save_state(LLMK_GPT2* m, const char* filename, int step);
 void gpt2_load_state(LLMK_GPT2* m, const char* filename, int* step);
+/* The same two under the reference's names and argument order, with the training data loader (llmk_data.h) whose
+ * position and, when it shuffles, permutations and generator go into / come out of the file (train_gpt2.cu:1228-1247,
+ * :1289-1310). loader may be NULL. For load_state the loader must have been initialised on the same shards. */
+void gpt2_save_state_with_loader(const char* filename, int step, LLMK_GPT2* model, struct LLMK_DataLoader* loader);
+void gpt2_load_state_with_loader(int* step, LLMK_GPT2* model, struct LLMK_DataLoader* loader, const char* filename);
 
 /* ---- accessors (the reference reads the struct fields directly) ---- */
 float gpt2_mean_loss(const LLMK_GPT2* m);

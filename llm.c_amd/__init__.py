@@ -1,7 +1,8 @@
 """Python host side of the MI355X kernel library for llm.c's GPT-2 training step.
 
 This module only binds the C ABI declared in include/llmk.h (kernel launchers, one per launcher of
-the reference's llmc/*.cuh) and include/llmk_gpt2.h (the host GPT-2 driver) through ctypes. There is
+the reference's llmc/*.cuh), include/llmk_gpt2.h (the host GPT-2 driver) and include/llmk_data.h (data loaders,
+learning-rate schedules, token decoder) through ctypes. There is
 no Python or CPU implementation of any operation here: if the shared library has not been built
 (python llm.c_amd/build.py), loading raises.
 
@@ -87,6 +88,8 @@ DRIVER_ABI = {
     "gpt2_free": (None, [vp]),
     "gpt2_save_state": (None, [vp, C.c_char_p, i32]),
     "gpt2_load_state": (None, [vp, C.c_char_p, ip]),
+    "gpt2_save_state_with_loader": (None, [C.c_char_p, i32, vp, vp]),
+    "gpt2_load_state_with_loader": (None, [ip, vp, vp, C.c_char_p]),
     "gpt2_mean_loss": (f32, [vp]),
     "gpt2_num_parameters": (sz, [vp]),
     "gpt2_get_config": (None, [vp, ip]),
@@ -102,6 +105,56 @@ DRIVER_ABI = {
     "gpt2_get_rng_state": (C.c_ulonglong, [vp]),
     "gpt2_set_rng_state": (None, [vp, C.c_ulonglong]),
     "gpt2_activation_bytes": (sz, [vp]),
+}
+
+
+# include/llmk_data.h: shard loader, evaluation loader, learning-rate schedules, token decoder (host only)
+u64p = C.POINTER(C.c_size_t)
+DATA_ABI = {
+    "dataloader_create": (vp, []),
+    "dataloader_init": (None, [vp, C.c_char_p, sz, sz, i32, i32, i32]),
+    "dataloader_reset": (None, [vp]),
+    "dataloader_load_batch": (None, [vp]),
+    "dataloader_next_batch": (None, [vp]),
+    "dataloader_resume": (None, [vp, sz, sz]),
+    "dataloader_free": (None, [vp]),
+    "dataloader_inputs": (ip, [vp]),
+    "dataloader_targets": (ip, [vp]),
+    "dataloader_num_tokens": (sz, [vp]),
+    "dataloader_num_shards": (sz, [vp]),
+    "dataloader_shard_num_samples": (sz, [vp]),
+    "dataloader_current_shard_idx": (sz, [vp]),
+    "dataloader_current_sample_idx": (sz, [vp]),
+    "dataloader_should_shuffle": (i32, [vp]),
+    "dataloader_get_shuffle_state": (sz, [vp, vp]),
+    "dataloader_set_shuffle_state": (sz, [vp, vp, sz]),
+    "evalloader_create": (vp, []),
+    "evalloader_init": (None, [vp, C.c_char_p, sz, sz, i32, i32]),
+    "evalloader_reset": (None, [vp]),
+    "evalloader_next_batch": (None, [vp]),
+    "evalloader_stat_losses": (i32, [vp, vp]),
+    "evalloader_free": (None, [vp]),
+    "evalloader_inputs": (ip, [vp]),
+    "evalloader_targets": (ip, [vp]),
+    "evalloader_mask": (C.POINTER(C.c_char), [vp]),
+    "evalloader_label": (ip, [vp]),
+    "evalloader_num_examples": (i32, [vp]),
+    "evalloader_num_batches": (i32, [vp]),
+    "evalloader_start_example_index": (i32, [vp]),
+    "evalloader_end_example_index": (i32, [vp]),
+    "evalloader_current_example_index": (i32, [vp]),
+    "lr_scheduler_create": (vp, []),
+    "lr_scheduler_init": (None, [vp, C.c_char_p, f32, i32, i32, f32]),
+    "get_learning_rate": (f32, [vp, i32]),
+    "lr_scheduler_free": (None, [vp]),
+    "tokenizer_create": (vp, []),
+    "tokenizer_init": (None, [vp, C.c_char_p]),
+    "tokenizer_decode": (vp, [vp, u32]),          # char* kept as an address: NULL is a valid answer
+    "safe_printf": (None, [C.c_char_p]),
+    "tokenizer_free": (None, [vp]),
+    "tokenizer_init_ok": (i32, [vp]),
+    "tokenizer_eot_token": (i32, [vp]),
+    "tokenizer_vocab_size": (u32, [vp]),
 }
 
 
@@ -127,7 +180,7 @@ def load(precision="bf16"):
         raise LibraryMissing(f"{path} not found: build it with `python llm.c_amd/build.py` "
                              "(there is no fallback implementation)")
     lib = C.CDLL(path)
-    for table in (KERNEL_ABI, DRIVER_ABI):
+    for table in (KERNEL_ABI, DRIVER_ABI, DATA_ABI):
         for name, (res, args) in table.items():
             fn = getattr(lib, name)   # AttributeError here = header and library disagree
             fn.restype = res

@@ -1,6 +1,6 @@
 """Builds the gfx950 shared libraries in-tree:  lib/libllmk_bf16.so  and  lib/libllmk_fp32.so.
 
-Each library = the HIP kernels (csrc/*.hip) + the host GPT-2 driver (driver/gpt2.cpp) compiled for
+Each library = the HIP kernels (csrc/*.hip) + the host GPT-2 driver and data path (driver/*.cpp) compiled for
 one storage precision, the way the reference builds one binary per PRECISION (reference
 Makefile:232-244). hipcc cross-compiles for gfx950, so this also runs on a machine without a GPU.
 
@@ -20,7 +20,7 @@ OBJDIR = os.path.join(HERE, "build")
 
 KERNEL_SOURCES = ["runtime.hip", "layernorm.hip", "gelu.hip", "encoder.hip", "classifier.hip", "optimizer.hip",
                   "gemm.hip", "attention.hip"]
-DRIVER_SOURCES = ["gpt2.cpp"]
+DRIVER_SOURCES = ["gpt2.cpp", "data.cpp"]
 
 # -packed-fp32-ops off: this toolchain's packed fp32 instructions are not trusted on this hardware pool
 # -amdgpu-mfma-vgpr-form: keep MFMA accumulators in ordinary VGPRs. The softmax between the two MFMA groups of the

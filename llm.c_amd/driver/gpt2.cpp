@@ -17,6 +17,7 @@
 
 #include "../../include/llmk.h"
 #include "../../include/llmk_gpt2.h"
+#include "../../include/llmk_data.h"
 #include "rand.hpp"
 
 #define hipCheck(expr)                                                                            \
@@ -642,23 +643,40 @@ void gpt2_free(LLMK_GPT2* m) {
     delete m;
 }
 
-void gpt2_save_state(LLMK_GPT2* m, const char* filename, int step) {
+void gpt2_save_state(LLMK_GPT2* m, const char* filename, int step) { gpt2_save_state_with_loader(filename, step, m, nullptr); }
+void gpt2_load_state(LLMK_GPT2* m, const char* filename, int* step) { gpt2_load_state_with_loader(step, m, nullptr, filename); }
+
+// save_state, train_gpt2.cu:1209: header, AdamW moments (+ master weights), and for a shuffling loader its
+// permutations and generator. Without a loader the loader fields of the header stay zero.
+void gpt2_save_state_with_loader(const char* filename, int step, LLMK_GPT2* m, LLMK_DataLoader* loader) {
     FILE* f = fopen(filename, "wb");
     if (!f) { fprintf(stderr, "Error: Failed to open file '%s'\n", filename); exit(EXIT_FAILURE); }
     int hdr[256];
     memset(hdr, 0, sizeof hdr);
-    hdr[0] = 20240527; hdr[1] = 1; hdr[2] = 1; hdr[3] = 0; hdr[4] = m->use_master_weights; hdr[5] = 0;
+    hdr[0] = 20240527; hdr[1] = 1; hdr[2] = 1; hdr[3] = 0; hdr[4] = m->use_master_weights;
+    hdr[5] = loader ? dataloader_should_shuffle(loader) : 0;
     hdr[10] = step;
     memcpy(&hdr[20], &m->rng_state, 8);
     memcpy(&hdr[22], &m->rng_state_last_update, 8);
+    if (loader) {
+        const size_t shard = dataloader_current_shard_idx(loader), sample = dataloader_current_sample_idx(loader);
+        memcpy(&hdr[30], &shard, sizeof(size_t));
+        memcpy(&hdr[32], &sample, sizeof(size_t));
+    }
     fwrite(hdr, sizeof(int), 256, f);
     device_to_file(f, m->m_memory, m->num_parameters * sizeof(float), m->stream);
     device_to_file(f, m->v_memory, m->num_parameters * sizeof(float), m->stream);
     if (m->use_master_weights) device_to_file(f, m->master_weights, m->num_parameters * sizeof(float), m->stream);
+    if (loader && dataloader_should_shuffle(loader)) {
+        std::vector<char> st(dataloader_get_shuffle_state(loader, nullptr));
+        dataloader_get_shuffle_state(loader, st.data());
+        fwrite(st.data(), 1, st.size(), f);
+    }
     fclose(f);
 }
 
-void gpt2_load_state(LLMK_GPT2* m, const char* filename, int* step) {
+// load_state, train_gpt2.cu:1250. The loader (already initialised on the same files) is put back where it was.
+void gpt2_load_state_with_loader(int* step, LLMK_GPT2* m, LLMK_DataLoader* loader, const char* filename) {
     FILE* f = fopen(filename, "rb");
     if (!f) { fprintf(stderr, "Error: Failed to open file '%s'\n", filename); exit(EXIT_FAILURE); }
     int hdr[256];
@@ -685,6 +703,20 @@ void gpt2_load_state(LLMK_GPT2* m, const char* filename, int* step) {
         gpt2_update(m, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0, 1);
     }
     m->rng_state = final_rng;
+    if (loader) {
+        if (hdr[5] == 1) {
+            const long at = ftell(f);
+            fseek(f, 0, SEEK_END);
+            std::vector<char> st((size_t)(ftell(f) - at));
+            fseek(f, at, SEEK_SET);
+            if (fread(st.data(), 1, st.size(), f) != st.size()) { fprintf(stderr, "Error: short read of the loader state\n"); exit(EXIT_FAILURE); }
+            dataloader_set_shuffle_state(loader, st.data(), st.size());
+        }
+        size_t shard, sample;
+        memcpy(&shard, &hdr[30], sizeof(size_t));
+        memcpy(&sample, &hdr[32], sizeof(size_t));
+        dataloader_resume(loader, shard, sample);
+    }
     fclose(f);
 }
 

@@ -54,6 +54,18 @@ public:
         }
     }
 
+    // The generator's state in the order of the reference's struct (llmc/rand.h:98-104, after its unused first field):
+    // left_, next_, the 624 state words. MATRIX_A there is the constant pair {0, 0x9908b0df}.
+    static constexpr uint32_t STATE_WORDS = 624;
+    void export_state(int32_t& left, uint32_t& next, uint32_t* words) const {
+        left = left_; next = (uint32_t)next_;
+        for (uint32_t j = 0; j < N; j++) words[j] = s_[j];
+    }
+    void import_state(int32_t left, uint32_t next, const uint32_t* words) {
+        left_ = left; next_ = (int)next;
+        for (uint32_t j = 0; j < N; j++) s_[j] = words[j];
+    }
+
 private:
     static constexpr uint32_t N = 624, M = 397;
     uint32_t s_[N];

@@ -14,6 +14,9 @@
 /* the sampler of the reference's GPU trainer (random_u32, random_f32, sample_softmax): a plain C header. The CPU
  * trainer's own copies of the first two sit behind #ifndef TESTING (train_gpt2.c:1046-1073), so nothing clashes. */
 #include "llmc/sampler.h"
+/* the learning-rate schedules: also a plain C header that train_gpt2.c does not pull in (the data loaders and the
+ * tokenizer it does, train_gpt2.c:25-29, so those are exported as they are) */
+#include "llmc/schedulers.h"
 
 /* Runs the reference's own gpt2_forward / gpt2_zero_grad / gpt2_backward / gpt2_update
  * (train_gpt2.c:1163-1169 call order) for `steps` steps on one fixed batch.
@@ -57,6 +60,89 @@ int ref_gpt2_generate(const char* ckpt, int* tokens, int T, int genT, int eot_to
     }
     gpt2_free(&model);
     return 0;
+}
+
+/* ---- flat entry points around the reference's structs for the data path ---------------------------------- */
+
+/* nbatches calls of dataloader_next_batch (llmc/dataloader.h:222): every batch's inputs and targets and the loader's
+ * position after it. With reset_every > 0, dataloader_reset is called before every reset_every-th batch (the way the
+ * trainer restarts the validation loader, train_gpt2.cu:1721). state_out (optional) receives the shuffle state in the
+ * order save_state writes it (train_gpt2.cu:1241-1247); returns its byte count. */
+size_t ref_dataloader_run(const char* pattern, size_t B, size_t T, int rank, int nproc, int shuffle, int nbatches,
+                          int reset_every, int* inputs_out, int* targets_out, size_t* shard_idx_out, size_t* sample_idx_out,
+                          size_t* num_tokens_out, void* state_out) {
+    DataLoader loader;
+    dataloader_init(&loader, pattern, B, T, rank, nproc, shuffle);
+    *num_tokens_out = loader.num_tokens;
+    for (int i = 0; i < nbatches; i++) {
+        if (reset_every > 0 && i > 0 && i % reset_every == 0) dataloader_reset(&loader);
+        dataloader_next_batch(&loader);
+        memcpy(inputs_out + (size_t)i * B * T, loader.inputs, B * T * sizeof(int));
+        memcpy(targets_out + (size_t)i * B * T, loader.targets, B * T * sizeof(int));
+        shard_idx_out[i] = loader.current_shard_idx;
+        sample_idx_out[i] = loader.current_sample_idx;
+    }
+    size_t bytes = 0;
+    if (shuffle && state_out) {
+        char* p = (char*)state_out;
+        memcpy(p, &loader.glob_result.gl_pathc, sizeof(size_t)); p += sizeof(size_t);
+        memcpy(p, loader.shard_indices, loader.glob_result.gl_pathc * sizeof(int)); p += loader.glob_result.gl_pathc * sizeof(int);
+        memcpy(p, &loader.shard_num_samples, sizeof(size_t)); p += sizeof(size_t);
+        memcpy(p, loader.intra_shard_indices, loader.shard_num_samples * sizeof(int)); p += loader.shard_num_samples * sizeof(int);
+        memcpy(p, &loader.shuffle_rng, sizeof(mt19937_state)); p += sizeof(mt19937_state);
+        bytes = (size_t)(p - (char*)state_out);
+    }
+    dataloader_free(&loader);
+    return bytes;
+}
+
+/* nbatches calls of evalloader_next_batch (llmc/dataloader.h:449) and evalloader_stat_losses on the given losses */
+int ref_evalloader_run(const char* filename, size_t B, size_t T, int rank, int nproc, int nbatches, int* inputs_out,
+                       int* targets_out, char* mask_out, int* label_out, const float* losses, int* correct_out, int* info_out) {
+    EvalLoader loader;
+    evalloader_init(&loader, filename, B, T, rank, nproc);
+    info_out[0] = loader.num_examples; info_out[1] = loader.num_batches;
+    info_out[2] = loader.start_example_index; info_out[3] = loader.end_example_index;
+    int can_fit = (int)(B / ASSUMED_NUM_COMPLETIONS);
+    for (int i = 0; i < nbatches; i++) {
+        evalloader_next_batch(&loader);
+        memcpy(inputs_out + (size_t)i * B * T, loader.inputs, B * T * sizeof(int));
+        memcpy(targets_out + (size_t)i * B * T, loader.targets, B * T * sizeof(int));
+        memcpy(mask_out + (size_t)i * B * T, loader.mask, B * T);
+        memcpy(label_out + (size_t)i * can_fit, loader.label, can_fit * sizeof(int));
+        correct_out[i] = evalloader_stat_losses(&loader, (float*)losses + (size_t)i * B * T);
+    }
+    info_out[4] = loader.current_example_index;
+    evalloader_free(&loader);
+    return 0;
+}
+
+/* get_learning_rate (llmc/schedulers.h:83) for steps 0..nsteps-1 */
+void ref_learning_rates(const char* type, float lr, int warmup, int num_batches, float final_frac, int nsteps, float* out) {
+    LearningRateScheduler s;
+    lr_scheduler_init(&s, type, lr, warmup, num_batches, final_frac);
+    for (int i = 0; i < nsteps; i++) out[i] = get_learning_rate(&s, i);
+}
+
+/* tokenizer_init + tokenizer_decode (llmc/tokenizer.h:41,86): the decoded bytes of ids[0..n) back to back into out
+ * (each followed by a 0 byte); returns the end-of-text id, or -1 when the file could not be opened */
+int ref_tokenizer_decode(const char* filename, const unsigned int* ids, int n, char* out, size_t out_bytes, unsigned int* vocab_out) {
+    Tokenizer t;
+    tokenizer_init(&t, filename);
+    if (!t.init_ok) return -1;
+    *vocab_out = t.vocab_size;
+    size_t o = 0;
+    for (int i = 0; i < n; i++) {
+        const char* sp = tokenizer_decode(&t, ids[i]);
+        size_t len = sp ? strlen(sp) : 0;
+        if (o + len + 1 > out_bytes) break;
+        if (sp) memcpy(out + o, sp, len);
+        out[o + len] = 0;
+        o += len + 1;
+    }
+    int eot = t.eot_token;
+    tokenizer_free(&t);
+    return eot;
 }
 
 int ref_num_threads(void) {

@@ -1,9 +1,11 @@
 """Writes tests/golden/tiny_gpt2.npz: what the reference's own CPU trainer (train_gpt2.c, compiled
-unmodified into oracle/_ref by oracle/Makefile) produces on a tiny seeded GPT-2, and
-tests/golden/tiny_gpt2_generate.npz: the tokens its forward pass and llmc/sampler.h generate from that model.
+unmodified into oracle/_ref by oracle/Makefile) produces on a tiny seeded GPT-2,
+tests/golden/tiny_gpt2_generate.npz: the tokens its forward pass and llmc/sampler.h generate from that model, and
+tests/golden/data_path.npz: the batches its data loaders (llmc/dataloader.h) serve from seeded synthetic files and the
+rates its schedules (llmc/schedulers.h) give.
 
 Run in the build container, where the reference checkout exists:
-    make -C oracle all _ref && python tests/golden/make_golden.py [train|generate]
+    make -C oracle all _ref && python tests/golden/make_golden.py [train|generate|data]
 The fixture holds data only: the configuration, the tokens, the per-step losses, and samples of
 the logits, gradients and updated parameters (indices + values), so that the oracle restatement
 and the GPU path can be checked against the reference on machines that do not have it.
@@ -42,12 +44,55 @@ def write_generate_fixture():
     print("tokens", tokens)
 
 
+def write_data_fixture():
+    import data_files as df
+    R = ol.ref()
+    sizes, vocab, shard_seed = [1000, 777, 1301], 50257, 11
+    B, T, rank, nproc, nb = 2, 8, 1, 2, 120
+    out = dict(shard_sizes=np.array(sizes), vocab=vocab, shard_seed=shard_seed, B=B, T=T, rank=rank, nproc=nproc, nbatches=nb)
+    with tempfile.TemporaryDirectory() as d:
+        pattern, _ = df.synthetic_shards(d, sizes, vocab, shard_seed)
+        for shuffle in (0, 1):
+            inp = np.zeros((nb, B * T), np.int32); tgt = np.zeros_like(inp)
+            si = np.zeros(nb, np.uint64); sa = np.zeros(nb, np.uint64)
+            ntok = C.c_size_t(0)
+            buf = C.create_string_buffer(1 << 16)
+            n = R.ref_dataloader_run(pattern.encode(), B, T, rank, nproc, shuffle, nb, 0, inp.reshape(-1), tgt.reshape(-1),
+                                     si, sa, C.byref(ntok), buf)
+            out[f"inputs_shuffle{shuffle}"], out[f"targets_shuffle{shuffle}"] = inp, tgt
+            out[f"pos_shuffle{shuffle}"] = np.stack([si, sa], 1)
+            if shuffle:
+                state = bytearray(buf.raw[:n])
+                cut = n - (8 + 4 + 4 + 624 * 4 + 8)
+                state[cut:cut + 8] = bytes(8)          # the generator's first field is never set by the reference
+                out["state_shuffle1"] = np.frombuffer(bytes(state), np.uint8)
+        eN, eseed, eB, eT, enb, lseed = 23, 12, 12, 40, 9, 13
+        path = os.path.join(d, "eval.bin")
+        df.write_eval_file(path, df.synthetic_eval_examples(eN, vocab, eseed))
+        losses = np.random.RandomState(lseed).rand(enb, eB * eT).astype(np.float32)
+        inp = np.zeros((enb, eB * eT), np.int32); tgt = np.zeros_like(inp)
+        mask = np.zeros((enb, eB * eT), np.int8); label = np.zeros((enb, eB // 4), np.int32)
+        correct = np.zeros(enb, np.int32); info = np.zeros(5, np.int32)
+        R.ref_evalloader_run(path.encode(), eB, eT, 0, 1, enb, inp.reshape(-1), tgt.reshape(-1), mask.reshape(-1),
+                             label.reshape(-1), losses.reshape(-1), correct, info)
+        out.update(eval_examples=eN, eval_seed=eseed, eval_B=eB, eval_T=eT, eval_nbatches=enb, eval_loss_seed=lseed,
+                   eval_inputs=inp, eval_targets=tgt, eval_mask=mask, eval_correct=correct)
+    for kind in ("cosine", "linear", "constant", "wsd"):
+        lrs = np.zeros(301, np.float32)
+        R.ref_learning_rates(kind.encode(), 6e-4, 20, 300, 0.1, 301, lrs)
+        out[f"lr_{kind}"] = lrs
+    np.savez_compressed(os.path.join(HERE, "data_path.npz"), **out)
+    print("data fixture: correct per eval batch", correct)
+
+
 def main():
     assert ol.have_ref(), "build oracle/_ref first (needs the reference checkout)"
-    which = sys.argv[1] if len(sys.argv) > 1 else "both"
-    if which in ("generate", "both"):
+    which = sys.argv[1] if len(sys.argv) > 1 else "all"
+    if which in ("generate", "all"):
         write_generate_fixture()
-    if which == "generate":
+    if which in ("data", "all"):
+        write_data_fixture()
+    if which in ("generate", "data"):
         return
     cfg = ol.Config(**CFG)
     params = ol.init_params(cfg, SEED)

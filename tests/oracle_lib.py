@@ -137,6 +137,16 @@ def ref():
     L.sample_softmax.restype = C.c_int
     L.ref_gpt2_generate.argtypes = [C.c_char_p, i32p, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_uint64)]
     L.ref_gpt2_generate.restype = C.c_int
+    szp = np.ctypeslib.ndpointer(dtype=np.uint64, flags="C_CONTIGUOUS")
+    L.ref_dataloader_run.argtypes = [C.c_char_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int,
+                                     i32p, i32p, szp, szp, C.POINTER(C.c_size_t), C.c_void_p]
+    L.ref_dataloader_run.restype = C.c_size_t
+    L.ref_evalloader_run.argtypes = [C.c_char_p, C.c_size_t, C.c_size_t, C.c_int, C.c_int, C.c_int, i32p, i32p,
+                                     np.ctypeslib.ndpointer(dtype=np.int8, flags="C_CONTIGUOUS"), i32p, f32p, i32p, i32p]
+    L.ref_evalloader_run.restype = C.c_int
+    L.ref_learning_rates.argtypes = [C.c_char_p, C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, f32p]
+    L.ref_tokenizer_decode.argtypes = [C.c_char_p, u32p, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint)]
+    L.ref_tokenizer_decode.restype = C.c_int
     L.ref_num_threads.restype = C.c_int
     _ref = L
     return L

@@ -9,10 +9,14 @@ import gpu_lib
 ROOT = gpu_lib.ROOT
 
 
-def declared(header):
+def declared(header, prefixes="llmk|gpt2"):
     src = open(os.path.join(ROOT, "include", header)).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return sorted(set(re.findall(r"\b((?:llmk|gpt2)_[a-z0-9_]+)\s*\(", src)))
+    return sorted(set(re.findall(r"\b((?:%s)_[a-z0-9_]+)\s*\(" % prefixes, src)))
+
+
+def declared_data():
+    return sorted(declared("llmk_data.h", "dataloader|evalloader|lr_scheduler|tokenizer|get_learning|safe") )
 
 
 @pytest.fixture(scope="module")
@@ -29,7 +33,7 @@ def pkg():
 @pytest.mark.parametrize("precision", ["bf16", "fp32"])
 def test_every_declared_symbol_is_exported(pkg, precision):
     L = pkg.load(precision)
-    names = declared("llmk.h") + declared("llmk_gpt2.h")
+    names = declared("llmk.h") + declared("llmk_gpt2.h") + declared_data()
     assert len(names) > 50
     missing = [n for n in names if not hasattr(L, n)]
     assert not missing, missing
@@ -40,6 +44,7 @@ def test_every_declared_symbol_is_exported(pkg, precision):
 def test_python_binding_tables_match_headers(pkg):
     assert sorted(pkg.KERNEL_ABI) == declared("llmk.h")
     assert sorted(pkg.DRIVER_ABI) == declared("llmk_gpt2.h")
+    assert sorted(pkg.DATA_ABI) == declared_data() and len(pkg.DATA_ABI) > 40
 
 
 def test_missing_library_raises(pkg, monkeypatch):

@@ -254,6 +254,57 @@ def test_checkpoint_and_state_resume_is_bit_identical(precision, tmp_path):
         m3.free()
 
 
+def test_training_loop_on_shards_resumes_bit_identical(tmp_path):
+    """The trainer's loop (train_gpt2.cu:1829-1852) with the library's shard loader and learning-rate schedule, and the
+    resume of test_gpt2.cu:326-367 with the loader's state in the state file (train_gpt2.cu:1228-1247, :1289-1310):
+    a run stopped after 4 steps and resumed sees the same batches and the same bits as the run that went on."""
+    import data_files as df
+    cfg = ol.Config(64, 300, 320, 2, 2, 128)
+    B, T, steps = 2, 64, 9
+    pattern, _ = df.synthetic_shards(str(tmp_path), [700, 900, 650], cfg.vocab_size, seed=21)   # 4-6 samples per shard
+    L = G.lib("bf16")
+
+    def make_loader():
+        h = L.dataloader_create()
+        L.dataloader_init(h, pattern.encode(), B, T, 0, 1, 1)
+        return h
+
+    sched = L.lr_scheduler_create()
+    L.lr_scheduler_init(sched, b"cosine", 3e-3, 2, steps, 0.1)
+
+    def run(m, loader, first, last):
+        out = []
+        for s in range(first, last):
+            L.dataloader_next_batch(loader)
+            inp = np.ctypeslib.as_array(L.dataloader_inputs(loader), shape=(B * T,)).copy()
+            tgt = np.ctypeslib.as_array(L.dataloader_targets(loader), shape=(B * T,)).copy()
+            out.append((m.step(inp, tgt, s + 1, L.get_learning_rate(sched, s), 0.9, 0.95, 1e-8, 0.1, clip=1.0),
+                        inp.tobytes(), L.dataloader_current_shard_idx(loader), L.dataloader_current_sample_idx(loader)))
+        return out
+
+    m, loader = Model("bf16", cfg, B, T, seed=9, master=1), make_loader()
+    run(m, loader, 0, 4)
+    ck, stt = str(tmp_path / "model.bin"), str(tmp_path / "state.bin")
+    L.gpt2_write_to_checkpoint(m.h, ck.encode())
+    L.gpt2_save_state_with_loader(stt.encode(), 4, m.h, loader)
+    first = run(m, loader, 4, steps)
+    p_first = m.params()
+    m.free(); L.dataloader_free(loader)
+    shdr = np.fromfile(stt, dtype=np.int32, count=256)
+    assert shdr[5] == 1 and shdr[10] == 4                   # the loader shuffles; the step
+    assert os.path.getsize(stt) > 1024 + 3 * 4 * sum(ol.param_sizes(cfg)[0]) + 2 * 8 + 3 * 4 + 2500
+    m2, loader2 = Model("bf16", cfg, B, T, master=1, checkpoint=ck, weight_init=0), make_loader()
+    step = C.c_int(0)
+    L.gpt2_load_state_with_loader(C.byref(step), m2.h, loader2, stt.encode())
+    assert step.value == 4
+    again = run(m2, loader2, 4, steps)
+    assert again == first
+    np.testing.assert_array_equal(m2.params(), p_first)
+    assert len({b for _, b, _, _ in first}) == len(first)    # different batches, over a shard boundary
+    assert len({s for _, _, s, _ in first}) > 1
+    m2.free(); L.dataloader_free(loader2); L.lr_scheduler_free(sched)
+
+
 def test_validate_matches_training_forward_loss():
     cfg = ol.Config(64, 300, 320, 2, 2, 128)
     B, T = 2, 64
