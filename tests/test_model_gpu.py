@@ -305,6 +305,40 @@ def test_training_loop_on_shards_resumes_bit_identical(tmp_path):
     m2.free(); L.dataloader_free(loader2); L.lr_scheduler_free(sched)
 
 
+def test_multiple_choice_eval_scores_like_the_oracle(tmp_path):
+    """The HellaSwag pass of the trainer (train_gpt2.cu:1724-1749): evaluation batches -> gpt2_validate -> per-token
+    losses -> evalloader_stat_losses, against the same count from the oracle's logits."""
+    import data_files as df
+    cfg = ol.Config(64, 300, 320, 2, 2, 128)
+    B, T = 8, 64
+    examples = df.synthetic_eval_examples(9, cfg.vocab_size, seed=31)
+    path = str(tmp_path / "eval.bin")
+    df.write_eval_file(path, examples)
+    params = np.ascontiguousarray(ol.init_params(cfg, 5) * np.float32(3), np.float32)   # scaled: rows differ clearly
+    m = Model("fp32", cfg, B, T, params=params, master=0)
+    L = m.L
+    ev = L.evalloader_create()
+    L.evalloader_init(ev, path.encode(), B, T, 0, 1)
+    assert L.evalloader_num_batches(ev) == 5
+    got = want = 0
+    for _ in range(L.evalloader_num_batches(ev)):
+        L.evalloader_next_batch(ev)
+        inp = np.ctypeslib.as_array(L.evalloader_inputs(ev), shape=(B * T,)).copy()
+        tgt = np.ctypeslib.as_array(L.evalloader_targets(ev), shape=(B * T,)).copy()
+        L.gpt2_validate(m.h, inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p), B, T)
+        got += L.evalloader_stat_losses(ev, L.gpt2_cpu_losses(m.h))
+        logits = np.zeros(B * T * cfg.padded_vocab_size, np.float32)
+        assert ol.cref().cref_gpt2_logits(C.byref(cfg), params, inp, B, T, logits) == 0
+        z = logits.reshape(B * T, -1)[:, :cfg.vocab_size].astype(np.float64)
+        lse = np.log(np.exp(z - z.max(1, keepdims=True)).sum(1)) + z.max(1)
+        losses = (lse - z[np.arange(B * T), tgt]).astype(np.float32)
+        np.testing.assert_allclose(np.ctypeslib.as_array(L.gpt2_cpu_losses(m.h), shape=(B * T,)), losses, rtol=1e-3, atol=1e-3)
+        want += L.evalloader_stat_losses(ev, losses.ctypes.data_as(C.c_void_p))
+    assert got == want and 0 <= got <= 9
+    L.evalloader_free(ev)
+    m.free()
+
+
 def test_validate_matches_training_forward_loss():
     cfg = ol.Config(64, 300, 320, 2, 2, 128)
     B, T = 2, 64
