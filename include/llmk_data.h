@@ -1,8 +1,8 @@
 /*
  * llmk_data.h — C ABI of the host-side pieces that feed the training step and consume its results:
- * the token-shard loader, the multiple-choice evaluation loader, the learning-rate schedules and the
- * token decoder. They are the reference's llmc/dataloader.h, llmc/schedulers.h and llmc/tokenizer.h
- * under their own function names, with the structs opaque (created and freed by the library) so that
+ * the token-shard loader, the multiple-choice evaluation loader, the learning-rate schedules, the
+ * token decoder, the outlier detector and the run log. They are the reference's llmc/dataloader.h,
+ * schedulers.h, tokenizer.h, outlier_detector.h and logger.h under their own function names, with the structs opaque (created and freed by the library) so that
  * C, C++ and ctypes callers share one layout. File formats are the reference's, byte for byte.
  * None of these functions touches the GPU.
  *
@@ -107,6 +107,30 @@ void tokenizer_free(LLMK_Tokenizer* tokenizer);
 int tokenizer_init_ok(const LLMK_Tokenizer* tokenizer);
 int tokenizer_eot_token(const LLMK_Tokenizer* tokenizer);
 uint32_t tokenizer_vocab_size(const LLMK_Tokenizer* tokenizer);
+
+/* ---- loss / gradient-norm outlier detector (llmc/outlier_detector.h) ---------------------------
+ * A window of the last 128 values with running sum and sum of squares in double. */
+typedef struct LLMK_OutlierDetector LLMK_OutlierDetector;
+LLMK_OutlierDetector* outlier_detector_create(void);
+/* init_detector, llmc/outlier_detector.h:26 */
+void init_detector(LLMK_OutlierDetector* detector);
+/* update_detector, llmc/outlier_detector.h:36: NaN until the window is full, then the z-score of new_value against
+ * the window that already contains it (0 when the window has no spread) */
+double update_detector(LLMK_OutlierDetector* detector, double new_value);
+void outlier_detector_free(LLMK_OutlierDetector* detector);
+
+/* ---- run log (llmc/logger.h): lines appended to <log_dir>/main.log by process 0 ------------------ */
+typedef struct LLMK_Logger LLMK_Logger;
+LLMK_Logger* logger_create(void);
+/* logger_init, llmc/logger.h:19: inactive when log_dir is NULL or process_rank != 0; resume == 0 empties the file */
+void logger_init(LLMK_Logger* logger, const char* log_dir, int process_rank, int resume);
+/* logger_log_eval, llmc/logger.h:34: "s:%d eval:%.4f" */
+void logger_log_eval(LLMK_Logger* logger, int step, float val);
+/* logger_log_val, llmc/logger.h:42: "s:%d tel:%.4f" */
+void logger_log_val(LLMK_Logger* logger, int step, float val_loss);
+/* logger_log_train, llmc/logger.h:50: "s:%d trl:%.4f lr:%.6f norm:%.2f" */
+void logger_log_train(LLMK_Logger* logger, int step, float train_loss, float learning_rate, float grad_norm);
+void logger_free(LLMK_Logger* logger);
 
 #ifdef __cplusplus
 }

@@ -155,6 +155,16 @@ DATA_ABI = {
     "tokenizer_init_ok": (i32, [vp]),
     "tokenizer_eot_token": (i32, [vp]),
     "tokenizer_vocab_size": (u32, [vp]),
+    "outlier_detector_create": (vp, []),
+    "init_detector": (None, [vp]),
+    "update_detector": (C.c_double, [vp, C.c_double]),
+    "outlier_detector_free": (None, [vp]),
+    "logger_create": (vp, []),
+    "logger_init": (None, [vp, C.c_char_p, i32, i32]),
+    "logger_log_eval": (None, [vp, i32, f32]),
+    "logger_log_val": (None, [vp, i32, f32]),
+    "logger_log_train": (None, [vp, i32, f32, f32, f32]),
+    "logger_free": (None, [vp]),
 }
 
 

@@ -1,8 +1,9 @@
 // Host-side data path around the training step: token shards in, evaluation batches in, learning rate per step,
-// token ids back to text. Re-hosts the reference's llmc/dataloader.h, llmc/schedulers.h and llmc/tokenizer.h behind
+// token ids back to text, z-scores of loss and gradient norm, the run log. Re-hosts the reference's llmc/dataloader.h,
+// schedulers.h, tokenizer.h, outlier_detector.h and logger.h behind
 // include/llmk_data.h (same function names, same file formats, same sequence of batches for the same files and
 // seed). Files are read with pread at 64-bit offsets (the reference seeks with an offset cast to int,
-// dataloader.h:214, which limits a shard to 2 GiB); nothing here touches the GPU.
+// dataloader.h:213, which limits a shard to 2 GiB); nothing here touches the GPU.
 #include "../../include/llmk_data.h"
 
 #include <fcntl.h>
@@ -563,5 +564,94 @@ void tokenizer_free(LLMK_Tokenizer* t) { delete t; }
 int tokenizer_init_ok(const LLMK_Tokenizer* t) { return t->init_ok; }
 int tokenizer_eot_token(const LLMK_Tokenizer* t) { return t->eot_token; }
 uint32_t tokenizer_vocab_size(const LLMK_Tokenizer* t) { return t->vocab_size; }
+
+}  // extern "C"
+
+// ---------------------------------------------------------------------------------------------------------------
+// outlier detector (llmc/outlier_detector.h) and run log (llmc/logger.h)
+
+struct LLMK_OutlierDetector {
+    static constexpr int WINDOW = 128;
+    double buffer[WINDOW];
+    int count = 0, index = 0;
+    double sum = 0.0, sum_sq = 0.0;
+};
+
+struct LLMK_Logger {
+    int active = 0;
+    std::string path;
+};
+
+namespace {
+
+void append_line(const LLMK_Logger* lg, const char* fmt, ...) {
+    if (lg->active != 1) return;
+    FILE* f = fopen(lg->path.c_str(), "a");
+    if (!f) die("Error: Failed to open file '%s'", lg->path.c_str());
+    va_list ap;
+    va_start(ap, fmt);
+    vfprintf(f, fmt, ap);
+    va_end(ap);
+    fclose(f);
+}
+
+}  // namespace
+
+extern "C" {
+
+LLMK_OutlierDetector* outlier_detector_create(void) {
+    LLMK_OutlierDetector* d = new LLMK_OutlierDetector();
+    init_detector(d);
+    return d;
+}
+
+void init_detector(LLMK_OutlierDetector* d) {
+    for (double& x : d->buffer) x = 0.0;
+    d->count = 0; d->index = 0; d->sum = 0.0; d->sum_sq = 0.0;
+}
+
+double update_detector(LLMK_OutlierDetector* d, double v) {
+    constexpr int W = LLMK_OutlierDetector::WINDOW;
+    if (d->count < W) {                    // still filling the window
+        d->buffer[d->count++] = v;
+        d->sum += v;
+        d->sum_sq += v * v;
+        return nan("");
+    }
+    const double old = d->buffer[d->index];   // the oldest value leaves, the new one takes its place
+    d->sum -= old;
+    d->sum_sq -= old * old;
+    d->buffer[d->index] = v;
+    d->sum += v;
+    d->sum_sq += v * v;
+    d->index = (d->index + 1) % W;
+    const double mean = d->sum / W;
+    const double std_dev = sqrt(d->sum_sq / W - mean * mean);
+    if (std_dev == 0.0) return 0.0;
+    return (v - mean) / std_dev;
+}
+
+void outlier_detector_free(LLMK_OutlierDetector* d) { delete d; }
+
+LLMK_Logger* logger_create(void) { return new LLMK_Logger(); }
+
+void logger_init(LLMK_Logger* lg, const char* log_dir, int process_rank, int resume) {
+    lg->active = 0;
+    if (log_dir == nullptr || process_rank != 0) return;   // only the first process writes
+    lg->active = 1;
+    lg->path = std::string(log_dir) + "/main.log";
+    if (resume == 0) {                                      // a fresh run starts from an empty file
+        FILE* f = fopen(lg->path.c_str(), "w");
+        if (!f) die("Error: Failed to open file '%s'", lg->path.c_str());
+        fclose(f);
+    }
+}
+
+void logger_log_eval(LLMK_Logger* lg, int step, float val) { append_line(lg, "s:%d eval:%.4f\n", step, val); }
+void logger_log_val(LLMK_Logger* lg, int step, float val_loss) { append_line(lg, "s:%d tel:%.4f\n", step, val_loss); }
+void logger_log_train(LLMK_Logger* lg, int step, float train_loss, float learning_rate, float grad_norm) {
+    append_line(lg, "s:%d trl:%.4f lr:%.6f norm:%.2f\n", step, train_loss, learning_rate, grad_norm);
+}
+void logger_free(LLMK_Logger* lg) { delete lg; }
 
 }  // extern "C"

@@ -17,6 +17,8 @@
 /* the learning-rate schedules: also a plain C header that train_gpt2.c does not pull in (the data loaders and the
  * tokenizer it does, train_gpt2.c:25-29, so those are exported as they are) */
 #include "llmc/schedulers.h"
+#include "llmc/outlier_detector.h"
+#include "llmc/logger.h"
 
 /* Runs the reference's own gpt2_forward / gpt2_zero_grad / gpt2_backward / gpt2_update
  * (train_gpt2.c:1163-1169 call order) for `steps` steps on one fixed batch.
@@ -143,6 +145,24 @@ int ref_tokenizer_decode(const char* filename, const unsigned int* ids, int n, c
     int eot = t.eot_token;
     tokenizer_free(&t);
     return eot;
+}
+
+/* update_detector (llmc/outlier_detector.h:36) over a series */
+void ref_detector_run(const double* values, int n, double* z_out) {
+    OutlierDetector d;
+    init_detector(&d);
+    for (int i = 0; i < n; i++) z_out[i] = update_detector(&d, values[i]);
+}
+
+/* one line of each kind through llmc/logger.h, n times */
+void ref_logger_run(const char* log_dir, int rank, int resume, int n, const float* vals) {
+    Logger lg;
+    logger_init(&lg, log_dir, rank, resume);
+    for (int i = 0; i < n; i++) {
+        logger_log_train(&lg, i, vals[4 * i], vals[4 * i + 1], vals[4 * i + 2]);
+        if (i % 3 == 0) logger_log_val(&lg, i, vals[4 * i + 3]);
+        if (i % 5 == 0) logger_log_eval(&lg, i, vals[4 * i + 3] * 0.01f);
+    }
 }
 
 int ref_num_threads(void) {

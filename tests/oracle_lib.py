@@ -147,6 +147,9 @@ def ref():
     L.ref_learning_rates.argtypes = [C.c_char_p, C.c_float, C.c_int, C.c_int, C.c_float, C.c_int, f32p]
     L.ref_tokenizer_decode.argtypes = [C.c_char_p, u32p, C.c_int, C.c_char_p, C.c_size_t, C.POINTER(C.c_uint)]
     L.ref_tokenizer_decode.restype = C.c_int
+    f64p = np.ctypeslib.ndpointer(dtype=np.float64, flags="C_CONTIGUOUS")
+    L.ref_detector_run.argtypes = [f64p, C.c_int, f64p]
+    L.ref_logger_run.argtypes = [C.c_char_p, C.c_int, C.c_int, C.c_int, f32p]
     L.ref_num_threads.restype = C.c_int
     _ref = L
     return L

@@ -16,7 +16,7 @@ def declared(header, prefixes="llmk|gpt2"):
 
 
 def declared_data():
-    return sorted(declared("llmk_data.h", "dataloader|evalloader|lr_scheduler|tokenizer|get_learning|safe") )
+    return sorted(declared("llmk_data.h", "dataloader|evalloader|lr_scheduler|tokenizer|get_learning|safe|outlier_detector|init|update|logger") )
 
 
 @pytest.fixture(scope="module")

@@ -341,6 +341,73 @@ def test_tokenizer_matches_compiled_reference(L, tmp_path):
     L.tokenizer_free(h)
 
 
+# ---- outlier detector and run log -----------------------------------------------------------------------------------
+
+def ours_z(L, values):
+    h = L.outlier_detector_create()
+    out = np.array([L.update_detector(h, float(v)) for v in values])
+    L.outlier_detector_free(h)
+    return out
+
+
+def test_outlier_detector_is_the_z_score_of_the_last_128(L):
+    v = np.random.RandomState(14).randn(400) * 3 + 10
+    v[300] = 80.0                                         # an outlier
+    z = ours_z(L, v)
+    assert np.isnan(z[:128]).all() and not np.isnan(z[128:]).any()
+    for i in (128, 129, 255, 300, 399):
+        w = v[i - 127:i + 1]                              # the window already holds the new value
+        np.testing.assert_allclose(z[i], (v[i] - w.mean()) / w.std(), rtol=1e-9)
+    assert z[300] > 8 and np.abs(np.delete(z[128:], 300 - 128)).max() < 5
+    assert (ours_z(L, np.full(200, 2.5))[128:] == 0).all()        # no spread: zero, not a division by zero
+
+
+@needs_ref
+def test_outlier_detector_matches_compiled_reference(L):
+    v = np.random.RandomState(15).rand(1000) * 4 + 1
+    want = np.zeros(1000)
+    ol.ref().ref_detector_run(v, 1000, want)
+    got = ours_z(L, v)
+    assert (np.isnan(got) == np.isnan(want)).all()
+    np.testing.assert_allclose(got[128:], want[128:], rtol=1e-10)
+
+
+def ours_log(L, directory, rank, resume, n, vals):
+    h = L.logger_create()
+    L.logger_init(h, directory.encode() if directory else None, rank, resume)
+    for i in range(n):
+        L.logger_log_train(h, i, *[float(x) for x in vals[4 * i:4 * i + 3]])
+        if i % 3 == 0:
+            L.logger_log_val(h, i, float(vals[4 * i + 3]))
+        if i % 5 == 0:
+            L.logger_log_eval(h, i, float(np.float32(vals[4 * i + 3]) * np.float32(0.01)))
+    L.logger_free(h)
+
+
+def test_logger_lines(L, tmp_path):
+    vals = np.array([3.14159, 6e-4, 1.2345, 2.5] * 3, np.float32)
+    ours_log(L, str(tmp_path), 0, 0, 3, vals)
+    assert open(tmp_path / "main.log").read() == ("s:0 trl:3.1416 lr:0.000600 norm:1.23\ns:0 tel:2.5000\ns:0 eval:0.0250\n"
+                                                 "s:1 trl:3.1416 lr:0.000600 norm:1.23\ns:2 trl:3.1416 lr:0.000600 norm:1.23\n")
+    ours_log(L, str(tmp_path), 0, 1, 1, vals)             # resuming appends
+    assert open(tmp_path / "main.log").read().count("\n") == 8
+    ours_log(L, str(tmp_path), 1, 0, 1, vals)             # other processes do not write (and do not empty the file)
+    assert open(tmp_path / "main.log").read().count("\n") == 8
+    ours_log(L, str(tmp_path), 0, 0, 1, vals)             # a fresh run starts over
+    assert open(tmp_path / "main.log").read().count("\n") == 3
+
+
+@needs_ref
+def test_logger_matches_compiled_reference(L, tmp_path):
+    vals = (np.random.RandomState(16).rand(4 * 17) * 10).astype(np.float32)
+    a, b = tmp_path / "a", tmp_path / "b"
+    a.mkdir(); b.mkdir()
+    for resume in (0, 1):
+        ours_log(L, str(a), 0, resume, 17, vals)
+        ol.ref().ref_logger_run(str(b).encode(), 0, resume, 17, vals)
+        assert open(a / "main.log", "rb").read() == open(b / "main.log", "rb").read()
+
+
 # ---- the committed fixture: what the compiled reference produced, for machines without it ---------------------------
 
 def test_data_path_reproduces_reference_fixture(L, tmp_path):
