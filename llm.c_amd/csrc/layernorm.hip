@@ -184,11 +184,12 @@ residual_kernel(floatX* __restrict__ out, const floatX* __restrict__ a, const fl
 // partial goes to scratch[block][2][C]; a second kernel adds the partials in block order, so
 // the result does not depend on scheduling (no atomics).
 // One workgroup per CU, as many waves as the accumulators leave room for: 12 (three per SIMD) up to NV = 2, where the
-// kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8 at NV = 3,
-// 4 beyond (at NV = 4, C = 1600, eight waves spill half of their accumulators).
-constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 3 ? 8 : 4; }
+// kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8 at NV = 3 and,
+// with one row in flight per wave instead of two, at NV = 4 (C = 1600); 4 beyond, also with one row in flight (two
+// rows of 7 or 8 vectors beside the accumulators do not fit 256 registers).
+constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 4 ? 8 : 4; }
 template <int NV>
-__global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : 1)
+__global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : NV <= 4 ? 2 : 1)
 ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
                    const floatX* __restrict__ inp, const floatX* __restrict__ weight,
                    const float* __restrict__ mean, const float* __restrict__ rstd, int N, int C) {
@@ -257,7 +258,14 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
             }
         }
     };
-    {
+    if constexpr (NV >= 4) {
+        // wide rows: one row in flight per wave leaves room for twice the waves
+        vecX g0[NV], x0[NV], d0[NV];
+        for (int row = wave; row < N; row += nwaves) {
+            load_row(row, g0, x0, d0);
+            process_row(row, mean[row], rstd[row], g0, x0, d0);
+        }
+    } else {
         vecX g0[NV], x0[NV], d0[NV], g1[NV], x1[NV], d1[NV];
         int row = wave;
         float m0 = 0.f, r0 = 0.f, m1 = 0.f, r1 = 0.f;
