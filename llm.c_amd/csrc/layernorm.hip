@@ -185,11 +185,12 @@ residual_kernel(floatX* __restrict__ out, const floatX* __restrict__ a, const fl
 // the result does not depend on scheduling (no atomics).
 // One workgroup per CU, as many waves as the accumulators leave room for: 12 (three per SIMD) up to NV = 2, where the
 // kernel needs 170 registers, two more than three waves per SIMD allow, hence the occupancy request; 8 at NV = 3 and,
-// with one row in flight per wave instead of two, at NV = 4 (C = 1600); 4 beyond, also with one row in flight (two
-// rows of 7 or 8 vectors beside the accumulators do not fit 256 registers).
-constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 4 ? 8 : 4; }
+// with one row in flight per wave instead of two, at NV = 4 and 5 (C = 1600 .. 2560); 4 beyond, also with one row in
+// flight (two rows of 7 or 8 vectors beside the accumulators do not fit 256 registers). At NV = 2, 16 waves with one
+// row each measured the same as 12 with two.
+constexpr int lnb_waves(int nv) { return nv <= 2 ? 12 : nv <= 5 ? 8 : 4; }
 template <int NV>
-__global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : NV <= 4 ? 2 : 1)
+__global__ void __launch_bounds__(lnb_waves(NV) * 64, NV <= 2 ? 3 : NV <= 5 ? 2 : 1)
 ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
                    const floatX* __restrict__ inp, const floatX* __restrict__ weight,
                    const float* __restrict__ mean, const float* __restrict__ rstd, int N, int C) {
@@ -226,7 +227,7 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
             }
         }
     };
-    auto process_row = [&](int row, float m, float r, const vecX (&g)[NV], const vecX (&x)[NV], const vecX (&di)[NV]) {
+    auto process_row = [&](int row, float m, float r, vecX (&g)[NV], vecX (&x)[NV], vecX (&di)[NV]) {
         const size_t base = (size_t)row * C;
         float a = 0.f, bsum = 0.f;
 #pragma unroll
@@ -241,6 +242,14 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
             }
         a = wave_sum(a) * invC;
         bsum = wave_sum(bsum) * invC;
+        // the row stays packed as loaded: converted columns carried over the reductions cost up to 50 registers
+#pragma unroll
+        for (int i = 0; i < NV; i++) {
+            unsigned* g32 = reinterpret_cast<unsigned*>(&g[i]);
+            unsigned* x32 = reinterpret_cast<unsigned*>(&x[i]);
+#pragma unroll
+            for (int q = 0; q < 4; q++) { asm volatile("" : "+v"(g32[q])); asm volatile("" : "+v"(x32[q])); }
+        }
 #pragma unroll
         for (int i = 0; i < NV; i++) {
             int v = lane + i * 64;
@@ -399,7 +408,7 @@ void llmk_layernorm_backward(void* dinp, void* dweight, void* dbias, float* scra
         static bool attr_set = false;                                                                        \
         if (!attr_set) {                                                                                     \
             HIP_CHECK(hipFuncSetAttribute((const void*)ln_backward_kernel<K>,                                \
-                                          hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024));          \
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));          \
             attr_set = true;                                                                                 \
         }                                                                                                    \
         ln_backward_kernel<K><<<blocks, lnb_waves(K) * 64, smem, st>>>((floatX*)dinp, scratch, (const floatX*)dout, \
