@@ -191,6 +191,13 @@ __device__ __forceinline__ void fa_block_coords(int& tile, int& bh) {
     }
 }
 
+// The running reference point m of a row (log2 units) only has to stay near the row's maximum, not at it: the
+// probabilities are exp2(s - m) and the final division by their sum takes m out again. Moving m costs 48 multiplies
+// per lane (output and row-sum accumulators), a fifth of the loop's vector work, and with m at the exact maximum some
+// row of the 32 moves in most steps. So a row's m follows its maximum only once a score exceeds m by FA_MAX_SLACK;
+// until then probabilities may reach 2^FA_MAX_SLACK instead of 1, which neither bf16 nor the fp32 sums mind.
+constexpr float FA_MAX_SLACK = 8.0f;
+
 // ---- forward ----------------------------------------------------------------------------------
 // grid (ceil(T/128), B*NH), 256 threads: wave w owns queries [128*qt + 32w, +32) and walks the key tiles up to
 // its diagonal, 32 keys at a time. The loop is bound by the vector ALU (one exp2 per score costs as much as the
@@ -307,9 +314,12 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
 #pragma unroll
             for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float m_new = fmaxf(m, mx * c);
-            if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // some row's running max moved: rescale (rare after the first tiles)
+            const float m_top = fmaxf(m, mx * c);
+            const bool outgrown = m_top > m + FA_MAX_SLACK;
+            if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
                 asm volatile("" ::: "memory");
+                // every row decides for itself, so that what a row computes depends on that row's scores alone
+                const float m_new = outgrown ? m_top : m;
                 const float alpha = fast_exp2(m - m_new);
                 m = m_new;
 #pragma unroll
@@ -437,9 +447,12 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
 #pragma unroll
             for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
             mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float m_new = fmaxf(m, mx * c);
-            if (__builtin_amdgcn_ballot_w64(m_new > m) != 0) {   // some row's running max moved: rescale (rare after the first tiles)
+            const float m_top = fmaxf(m, mx * c);
+            const bool outgrown = m_top > m + FA_MAX_SLACK;
+            if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
                 asm volatile("" ::: "memory");
+                // every row decides for itself, so that what a row computes depends on that row's scores alone
+                const float m_new = outgrown ? m_top : m;
                 const float alpha = fast_exp2(m - m_new);
                 m = m_new;
 #pragma unroll
