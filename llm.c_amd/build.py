@@ -1,4 +1,5 @@
-"""Builds the gfx950 shared libraries in-tree:  lib/libllmk_bf16.so  and  lib/libllmk_fp32.so.
+"""Builds the gfx950 shared libraries in-tree:  lib/libllmk_bf16.so  and  lib/libllmk_fp32.so, and the trainer
+programs lib/train_gpt2_bf16 and lib/train_gpt2_fp32 linked against them.
 
 Each library = the HIP kernels (csrc/*.hip) + the host GPT-2 driver and data path (driver/*.cpp) compiled for
 one storage precision, the way the reference builds one binary per PRECISION (reference
@@ -34,6 +35,10 @@ def lib_path(precision):
     return os.path.join(LIBDIR, f"libllmk_{precision}.so")
 
 
+def trainer_path(precision):
+    return os.path.join(LIBDIR, f"train_gpt2_{precision}")
+
+
 def _run(cmd):
     r = subprocess.run(cmd, capture_output=True, text=True)
     out = "\n".join(l for l in (r.stdout + r.stderr).splitlines()
@@ -67,6 +72,9 @@ def build(precisions=("bf16", "fp32"), jobs=8, verbose=False):
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", lib_path(p), *objs[p]])
         if verbose:
             print("built", lib_path(p))
+        # the trainer program (the reference's main loop) against that library; found next to it at run time
+        _run([hipcc, "-O2", "-std=c++17", "-Wall", "-x", "hip", "--offload-arch=gfx950", os.path.join(DRIVER, "train_gpt2.cpp"),
+              "-o", trainer_path(p), "-L" + LIBDIR, f"-lllmk_{p}", "-Wl,-rpath,$ORIGIN"])
     return [lib_path(p) for p in precisions]
 
 

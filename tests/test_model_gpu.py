@@ -305,6 +305,46 @@ def test_training_loop_on_shards_resumes_bit_identical(tmp_path):
     m2.free(); L.dataloader_free(loader2); L.lr_scheduler_free(sched)
 
 
+def test_trainer_program_trains_checkpoints_and_resumes(tmp_path):
+    """The trainer program (the reference's main loop, train_gpt2.cu:1419-1900, against the C ABI) on synthetic shards:
+    validation, sampling, log lines, checkpoint files, and a resumed run (-y 1) that repeats the interrupted steps
+    with the same numbers."""
+    import glob
+    import re
+    import subprocess
+    import data_files as df
+    exe = os.path.join(G.ROOT, "llm.c_amd", "lib", "train_gpt2_bf16")
+    assert os.path.exists(exe), "build the library first (python llm.c_amd/build.py)"
+    data = tmp_path / "data"; data.mkdir()
+    train, _ = df.synthetic_shards(str(data), [3000, 2500], 50257, seed=41, prefix="train")
+    val, _ = df.synthetic_shards(str(data), [1500], 50257, seed=42, prefix="val")
+    log = tmp_path / "log"
+    args = [exe, "-i", train, "-j", val, "-e", "d6", "-o", str(log), "-b", "4", "-t", "64", "-x", "6", "-v", "3", "-m", "2",
+            "-s", "3", "-g", "8", "-n", "3", "-l", "1e-3", "-u", "2", "-q", "0.1", "-k", "linear"]
+    r = subprocess.run(args, capture_output=True, text=True, timeout=240, cwd=str(tmp_path))
+    assert r.returncode == 0, r.stdout[-2000:] + r.stderr[-2000:]
+    assert "step    6/6" in r.stdout and r.stdout.count("val loss") == 3 and r.stdout.count("generating:") == 2
+    for step in (3, 6):
+        for name in (f"model_{step:08d}.bin", f"state_{step:08d}_00000.bin", f"DONE_{step:08d}"):
+            assert (log / name).exists(), name
+    lines = open(log / "main.log").read().split("\n")
+    trl = {int(m.group(1)): m.group(0) for m in (re.match(r"s:(\d+) trl:.*", l) for l in lines) if m}
+    assert sorted(trl) == [0, 1, 2, 3, 4, 5]
+    lrs = [float(re.search(r"lr:([0-9.]+)", trl[s]).group(1)) for s in range(6)]
+    assert lrs[0] == 0.0005 and lrs[1] == 0.001 and lrs[5] < lrs[2]       # warm-up over two steps, then decay
+    assert sum("tel:" in l for l in lines) == 3
+    # interrupt after step 3: drop what came later, resume, and the steps 4-6 come out the same
+    for f in glob.glob(str(log / "*00000006*")):
+        os.remove(f)
+    r2 = subprocess.run(args + ["-y", "1"], capture_output=True, text=True, timeout=240, cwd=str(tmp_path))
+    assert r2.returncode == 0, r2.stdout[-2000:] + r2.stderr[-2000:]
+    assert "step    4/6" in r2.stdout and "step    3/6" not in r2.stdout
+    lines2 = open(log / "main.log").read().split("\n")
+    resumed = [l for l in lines2[len(lines) - 1:] if re.match(r"s:\d+ trl:", l)]
+    assert resumed == [trl[3], trl[4], trl[5]]
+    assert (log / "DONE_00000006").exists()
+
+
 def test_multiple_choice_eval_scores_like_the_oracle(tmp_path):
     """The HellaSwag pass of the trainer (train_gpt2.cu:1724-1749): evaluation batches -> gpt2_validate -> per-token
     losses -> evalloader_stat_losses, against the same count from the oracle's logits."""
