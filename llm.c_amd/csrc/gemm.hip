@@ -597,8 +597,21 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
     hipStream_t st = (hipStream_t)stream;
     const int num_cu = llmk::device_info().num_cu;
 
-    // (1) dbias += column sums of dout
+    // The weight-gradient GEMM below reads dout as its K-major A operand; when it is the direct-to-LDS split-K kernel
+    // it adds up the rows of that operand on the side (EPI_PARTIAL_ROWSUM), which is the bias gradient without another
+    // pass over dout. Same preconditions as that kernel; otherwise the streaming reduction in (1).
+    bool dbias_in_gemm = false;
+#if !defined(LLMK_FP32)
     if (dbias) {
+        GemmArgs t{};
+        t.A = (const floatX*)dout; t.B = (const floatX*)inp; t.C = (floatX*)dweight;
+        t.M = OC; t.N = C; t.K = M; t.lda = OC; t.ldb = C; t.ldc = C; t.k_per_split = KGRAN;
+        dbias_in_gemm = pipelined_ok(t) && M % K_STEP == 0;
+    }
+#endif
+
+    // (1) dbias += column sums of dout
+    if (dbias && !dbias_in_gemm) {
         LLMK_REQUIRE(dbias_buffer != nullptr, "matmul_backward: dbias_buffer is required when dbias is given");
         const int ny = bias_grad_ny(OC);
         llmk::ProfScope prof("bias_grad", 0, (double)M * OC * sizeof(floatX), st);
@@ -669,14 +682,28 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         g.k_per_split = steps_per * K_STEP;
         const double tn_bytes = ((double)M * OC + (double)M * C + 2.0 * OC * C) * sizeof(floatX);
         if (splits == 1 && !tn_partial_always(g)) {
+            LLMK_REQUIRE(!dbias_in_gemm, "matmul_backward: bias gradient was left to a kernel that is not being run");
             llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
             launch_best<true, true, EPI_ACCUM>(g, 1, big, st);
         } else {
             const size_t mn = (size_t)OC * C;
-            g.partial = (float*)llmk::workspace(mn * splits * sizeof(float));
+            const int parts = big ? 4 : 2;                        // column waves of the tile configuration: each leaves a partial
+            g.partial = (float*)llmk::workspace((mn + (dbias_in_gemm ? (size_t)OC * parts : 0)) * splits * sizeof(float));
             {
                 llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
+#if !defined(LLMK_FP32)
+                if (dbias_in_gemm) {
+                    LLMK_REQUIRE(pipelined_ok(g), "matmul_backward: split of K (%d) does not suit the direct-to-LDS kernel", g.k_per_split);
+                    g.rowsum = g.partial + mn * splits;           // [splits * parts][OC]
+                    launch_pipelined<true, true, EPI_PARTIAL_ROWSUM>(g, splits, big, st);
+                } else
+#endif
                 launch_best<true, true, EPI_PARTIAL>(g, splits, big, st);
+            }
+            if (dbias_in_gemm) {                                  // dbias += the splits' row sums, in split order
+                llmk::ProfScope prof("bias_grad_reduce", 0, (double)splits * parts * OC * sizeof(float), st);
+                bias_grad_reduce_kernel<<<CEIL_DIV(OC, BGR_COLS), BGR_COLS * BGR_GROUPS, 0, st>>>((floatX*)dbias, g.rowsum, OC, splits * parts);
+                LAUNCH_CHECK();
             }
             llmk::ProfScope prof("splitk_reduce", 0, (double)mn * splits * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
             splitk_reduce_kernel<true><<<(unsigned)CEIL_DIV(mn / 4, (size_t)256), 256, 0, st>>>((floatX*)dweight, g.partial, mn, splits);

@@ -41,7 +41,9 @@ typedef __attribute__((ext_vector_type(16))) float f32x16;
 typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
-enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5 };
+// EPI_PARTIAL_ROWSUM: EPI_PARTIAL plus, per row m of the output, the sum over the split's K range of A(m, k): with
+// A = dout^T that is the bias gradient, taken from the operand fragments the matrix cores are being fed anyway.
+enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5, EPI_PARTIAL_ROWSUM = 6 };
 
 struct GemmArgs {
     const floatX* A;
@@ -51,7 +53,8 @@ struct GemmArgs {
     int lda, ldb, ldc;    // leading dimensions of the stored matrices, in elements
     const floatX* bias;   // [N] or nullptr                         (EPI_BIAS*)
     floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU)
-    float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL)
+    float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL*)
+    float* rowsum;        // [splits * ROWSUM_PARTS][M] fp32        (EPI_PARTIAL_ROWSUM)
     int k_per_split;      // multiple of the K block
     int splits;
 };
@@ -129,7 +132,10 @@ gemm_pipelined_kernel(GemmArgs g) {
     constexpr int WTM = BM / WGM, WTN = BN / WGN, TM = WTM / 32, TN = WTN / 32;
     constexpr int A_STAGE = BM * PBK * 2, B_STAGE = BN * PBK * 2, STAGE = A_STAGE + B_STAGE;
     constexpr int A_CHUNKS = A_STAGE / 1024, B_CHUNKS = B_STAGE / 1024;
-    constexpr int PASSES_OF_EPI = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
+    constexpr bool IS_PARTIAL = (EPI == EPI_PARTIAL || EPI == EPI_PARTIAL_ROWSUM);
+    constexpr bool ROWSUM = (EPI == EPI_PARTIAL_ROWSUM);
+    static_assert(!ROWSUM || A_T, "row sums are taken from K-major A fragments");
+    constexpr int PASSES_OF_EPI = (IS_PARTIAL || EPI == EPI_ACCUM) ? TN : TN / 2;   // epilogue passes over a 32-row block
     constexpr int CPW = (A_CHUNKS + B_CHUNKS) / NW;            // 1 KiB chunks each wave requests per K block
     static_assert((A_CHUNKS + B_CHUNKS) % NW == 0, "chunks must divide evenly over the waves");
     constexpr bool TR_ASM = (A_T && B_T) ? LLMK_TR_ASM_BOTH : LLMK_TR_ASM_MIXED;   // hand-issued or compiler-issued transposing reads
@@ -317,12 +323,32 @@ gemm_pipelined_kernel(GemmArgs g) {
     using Younger = std::integral_constant<int, TR_READS>;
     using NoneYounger = std::integral_constant<int, 0>;
     f32x16 acc[TM][TN];
-    auto mma = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN]) {
+    // Row sums of A (EPI_PARTIAL_ROWSUM): in the swapped MFMA the A fragment is the second operand, so lane l of
+    // fa[i] holds eight consecutive k of row i*32 + l%32 (k half l/32): a dot product with ones per pair adds them up.
+    // The WGN column waves of a row of waves hold the same fragments: they share the work by K, wave wn taking the
+    // 16-wide steps s of every stage with s % WGN == wn (one wave-uniform test per step), and only in the first tile
+    // column. Each wave writes its own partial, so there are splits * WGN of them per row, added up by the caller.
+    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+    float rsum[ROWSUM ? TM : 1];
+    int rowsum_step = -1;                  // the step of a stage this wave sums in the current tile, or none
+    auto mma = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN], auto step) {
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
             for (int j = 0; j < TN; j++)   // swapped operands: acc[i][j] = D^T block, rows = n, cols = m
                 acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[j], fa[i], acc[i][j], 0, 0, 0);
+        if constexpr (ROWSUM) {
+            if (rowsum_step == decltype(step)::value % WGN) {     // wave-uniform
+                const bf16x2 ones2 = {(__bf16)1.0f, (__bf16)1.0f};
+#pragma unroll
+                for (int i = 0; i < TM; i++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const bf16x2 pr = {fa[i][2 * e], fa[i][2 * e + 1]};
+                        rsum[i] = __builtin_amdgcn_fdot2_f32_bf16(pr, ones2, rsum[i], false);
+                    }
+            }
+        }
     };
     // Waiting for loads: vector-memory operations retire in issue order, so "at most N outstanding" means that
     // everything but the N youngest has landed. The stages of a tile are requested one at a time, so the only
@@ -347,7 +373,7 @@ gemm_pipelined_kernel(GemmArgs g) {
 
     // Epilogues that read global memory (the pre-GELU activations, the old weight gradient) request it while the
     // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
-    constexpr bool F32OUT = (EPI == EPI_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
+    constexpr bool F32OUT = (IS_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
     constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
     static_assert(EPI != EPI_DGELU, "GELU backward is not fused into this kernel");
     constexpr bool EPI_READS = (EPI == EPI_ACCUM);
@@ -410,6 +436,11 @@ gemm_pipelined_kernel(GemmArgs g) {
             for (int j = 0; j < TN; j++)
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        if constexpr (ROWSUM) {
+            rowsum_step = tile_n == 0 ? wn : -1;
+#pragma unroll
+            for (int i = 0; i < TM; i++) rsum[i] = 0.f;
+        }
 
         // ---- K loop over stages of 64, software-pipelined: the operands of the next 16-wide step (and the
         // barrier that publishes the next stage) are requested while the matrix cores work on the current step.
@@ -426,7 +457,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
-        constexpr bool EARLY0 = EPI != EPI_ACCUM && EPI != EPI_PARTIAL;
+        constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
         int next_kbeg = 0, next_nkb = 0;
         bool early0 = false;
         if (have_next) {
@@ -445,14 +476,14 @@ gemm_pipelined_kernel(GemmArgs g) {
             const unsigned cur = buf_of(st);
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0);
+            mma(fa0, fb0, S0{});
             if (late && st >= 1) issue(st + 1, buf_idx(st + 1));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1);
+            mma(fa1, fb1, S1{});
             read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0);
+            mma(fa0, fb0, S2{});
             __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
             if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
             barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
@@ -462,7 +493,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             }
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1);
+            mma(fa1, fb1, S3{});
         }
         {
             const unsigned cur = buf_of(nst - 1);
@@ -470,23 +501,33 @@ gemm_pipelined_kernel(GemmArgs g) {
             prefetch_epilogue(m0, n0, 0);
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0);
+            mma(fa0, fb0, S0{});
             if (EARLY0 && !HAS_BIAS && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1);
+            mma(fa1, fb1, S1{});
             bias_ready();                                         // two 16-wide steps after the request
             if (EARLY0 && HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
             read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0);
+            mma(fa0, fb0, S2{});
             await_frags(fa1, fb1, NoneYounger{});
-            mma(fa1, fb1);
+            mma(fa1, fb1, S3{});
         }
 
         // ---- request the next work item's first K blocks, then run the epilogue under them --------
         barrier_no_fence();                                  // every wave is done reading both buffers
         const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
+        if constexpr (ROWSUM) {
+            if (rowsum_step >= 0) {                               // the two k halves of a row sit 32 lanes apart
+#pragma unroll
+                for (int i = 0; i < TM; i++) {
+                    const float s = rsum[i] + __shfl_xor(rsum[i], 32, 64);
+                    const int m = cur_m0 + wm * WTM + i * 32 + idx;
+                    if (half == 0 && m < g.M) g.rowsum[((size_t)cur_split * WGN + wn) * g.M + m] = s;
+                }
+            }
+        }
         prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
         it++;
         if (have_next) {
@@ -566,7 +607,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                         if (F32OUT) {
                             const int n = wn0 + pass * 32 + ch * 4;
                             if (m < g.M && n < g.N) {
-                                if (EPI == EPI_PARTIAL) {
+                                if (IS_PARTIAL) {
                                     st_cached(reinterpret_cast<u32x4*>(g.partial + ((size_t)cur_split * g.M + m) * g.N + n), raw);
                                 } else {
                                     union { u32x4 u; f32x4 f; } x;

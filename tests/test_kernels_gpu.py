@@ -313,7 +313,10 @@ def test_matmul_forward_gelu(precision, fusion, M, Cc, OC):
                                            (32768, 768, 768, True),        # dinp on the 256x256 kernel with XCD-private row panels
                                            (2048, 1600, 6400, True),       # GPT-2 1558M fc
                                            (4096, 1600, 1600, True),       # odd number of 64-wide K stages in dinp
-                                           (16384, 832, 1600, False)])     # odd stage counts on the 256x256 kernel
+                                           (16384, 832, 1600, False),      # odd stage counts on the 256x256 kernel
+                                           (1024, 256, 384, True),         # bias gradient inside the dweight GEMM, 128x128 tiles
+                                           (1024, 192, 136, True),         # ... with output rows past the matrix edge
+                                           (4096, 768, 2440, True)])       # ... 256x256 tiles with a ragged last row of tiles
 def test_matmul_backward(precision, M, Cc, OC, bias):
     L = G.lib(precision)
     x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
