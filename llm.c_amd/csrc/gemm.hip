@@ -631,21 +631,21 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
 #if defined(LLMK_FP32)
         const bool fused = pre_gelu && gelu_fusion >= 2;
 #else
-        // bf16: gelu' in the epilogue costs the matrix cores more idle time than the extra elementwise pass takes
-        // (0.57 ms either way at (65536, 3072) on MI355X), so the GEMM stays plain and GELU backward runs after it.
-        const bool fused = false;
-        (void)gelu_fusion;
+        // bf16: gelu' goes into the epilogue of the direct-to-LDS kernel (big tiles only); the bias gradient of the layer
+        // below then comes out of its weight-gradient GEMM, and no elementwise pass over (B,T,4C) is left
+        const bool fused = pre_gelu && gelu_fusion >= 2 && big && aligned16(pre_gelu) && pipelined_ok(g);
 #endif
         {
             llmk::ProfScope prof(fused ? "gemm_nn_dgelu" : "gemm_nn", 2.0 * M * (double)OC * C,
                                  ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
-#if defined(LLMK_FP32)
             if (fused) {
                 g.aux = (floatX*)pre_gelu;
+#if defined(LLMK_FP32)
                 launch_best<false, true, EPI_DGELU>(g, 1, big, st);
-            } else
+#else
+                launch_pipelined_cfg<256, 256, 2, 4, false, true, EPI_DGELU>(g, 1, st);
 #endif
-            {
+            } else {
                 launch_best<false, true, EPI_STORE>(g, 1, big, st);
             }
         }

@@ -375,12 +375,25 @@ gemm_pipelined_kernel(GemmArgs g) {
     // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
     constexpr bool F32OUT = (IS_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
     constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
-    static_assert(EPI != EPI_DGELU, "GELU backward is not fused into this kernel");
-    constexpr bool EPI_READS = (EPI == EPI_ACCUM);
+    constexpr bool EPI_READS = (EPI == EPI_ACCUM || EPI == EPI_DGELU);
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
+    // GELU backward: the pre-activation values of the 16 bytes each lane stores per (block, pass, quarter), as it stores them
+    u32x4 pre_act[EPI == EPI_DGELU ? TM : 1][EPI == EPI_DGELU ? PASSES : 1][4];
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
         if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
+        if constexpr (EPI == EPI_DGELU) {
+#pragma unroll
+            for (int pass = 0; pass < PASSES; pass++)
+#pragma unroll
+                for (int t = 0; t < 4; t++) {
+                    const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                    const int m = wm0 + i * 32 + row;
+                    const int n = wn0 + pass * 64 + ch * 8;
+                    if (m < g.M && n < g.N) pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(g.aux + (size_t)m * g.ldc + n);
+                }
+            return;
+        }
 #pragma unroll
         for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
@@ -457,7 +470,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
-        constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
+        constexpr bool EARLY0 = EPI != EPI_ACCUM && EPI != EPI_DGELU && !IS_PARTIAL;
         int next_kbeg = 0, next_nkb = 0;
         bool early0 = false;
         if (have_next) {
@@ -629,6 +642,13 @@ gemm_pipelined_kernel(GemmArgs g) {
                                     st_out(reinterpret_cast<u32x4*>(g.aux + o), x.u);
 #pragma unroll
                                     for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
+                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                } else if (EPI == EPI_DGELU) {
+                                    // the product of the rounded gradient and gelu'(pre), as gelu_backward_inplace forms it
+                                    union { u32x4 u; bf16x8 h; } pa;
+                                    pa.u = pre_act[EPI == EPI_DGELU ? i : 0][EPI == EPI_DGELU ? pass : 0][t];
+#pragma unroll
+                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)pa.h[e]) * (float)x.h[e]);
                                     st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                 } else {
                                     st_out(reinterpret_cast<u32x4*>(g.C + o), x.u);

@@ -541,15 +541,11 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
         float* l_att = a.att + l * B * NH * T;
 
         if (R >= 1) llmk_gelu_forward(l_fch_gelu, l_fch_pre_gelu, (int)(B * T * 4 * C), st);
-        if (m->gelu_fusion >= 2) {
-            // GELU backward shares its pass over (B,T,4C) with the bias gradient of the fc layer, whose dout it produces
-            llmk_matmul_backward(dl_bt4c, dl_fcprojw, dl_fcprojb, dresidual, l_fch_gelu, l_fcprojw, scratchF, (int)B, (int)T, (int)(4 * C), (int)C, st, nullptr, 1);
-            llmk_gelu_backward_bias(dl_bt4c, l_fch_pre_gelu, dl_fcb, scratchF, (int)B, (int)T, (int)(4 * C), st);
-        } else {
-            llmk_matmul_backward(dl_bt4c, dl_fcprojw, dl_fcprojb, dresidual, l_fch_gelu, l_fcprojw, scratchF, (int)B, (int)T, (int)(4 * C), (int)C, st, l_fch_pre_gelu, m->gelu_fusion);
-        }
+        // with gelu_fusion 2 the GELU backward is the epilogue of this GEMM's dinp; the bias gradient of the fc layer, whose
+        // dout that produces, comes out of the fc weight-gradient GEMM below
+        llmk_matmul_backward(dl_bt4c, dl_fcprojw, dl_fcprojb, dresidual, l_fch_gelu, l_fcprojw, scratchF, (int)B, (int)T, (int)(4 * C), (int)C, st, l_fch_pre_gelu, m->gelu_fusion);
         if (R >= 2) llmk_layernorm_forward(l_ln2, l_ln2_mean, l_ln2_rstd, l_residual2, l_ln2w, l_ln2b, (int)B, (int)T, (int)C, st);
-        llmk_matmul_backward(dl_btc, dl_fcw, m->gelu_fusion >= 2 ? nullptr : dl_fcb, dl_bt4c, l_ln2, l_fcw, scratchF, (int)B, (int)T, (int)C, (int)(4 * C), st, nullptr, 1);
+        llmk_matmul_backward(dl_btc, dl_fcw, dl_fcb, dl_bt4c, l_ln2, l_fcw, scratchF, (int)B, (int)T, (int)C, (int)(4 * C), st, nullptr, 1);
         llmk_layernorm_backward(dresidual, dl_ln2w, dl_ln2b, scratchF, dl_btc, l_residual2, l_ln2w, l_ln2_mean, l_ln2_rstd, (int)B, (int)T, (int)C, st);
         llmk_matmul_backward(dl_btc, dl_attprojw, dl_attprojb, dresidual, l_atty, l_attprojw, scratchF, (int)B, (int)T, (int)C, (int)C, st, nullptr, 1);
         llmk_attention_backward(dl_bt4c, dl_btc, l_qkvr, l_atty, l_att, (int)B, (int)T, (int)NH, (int)C, st);

@@ -346,9 +346,11 @@ def test_matmul_backward(precision, M, Cc, OC, bias):
 
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("fusion", [0, 2])
-def test_matmul_backward_gelu(precision, fusion):
-    L = G.lib(precision)
-    M, Cc, OC = 320, 512, 128           # dinp has the 4C width: (M, Cc) with pre_gelu of the same shape
+@pytest.mark.parametrize("M,Cc,OC", [(320, 512, 128),        # few tiles: GELU backward as a pass of its own
+                                     (8192, 2048, 512),      # a tile per CU and more: in the GEMM's epilogue (bf16, fusion 2)
+                                     (8448, 2056, 192)])     # ... with ragged last tiles in both directions
+def test_matmul_backward_gelu(precision, fusion, M, Cc, OC):
+    L = G.lib(precision)                # dinp has the 4C width: (M, Cc) with pre_gelu of the same shape
     x, w = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision)
     g, pre = G.rounded(rnd((M, OC), 2), precision), G.rounded(rnd((M, Cc), 3, 2.0), precision)
     lin = G.rounded((g.astype(np.float64) @ w.astype(np.float64)).astype(np.float32), precision)
