@@ -425,10 +425,31 @@ void launch_best(const GemmArgs& g, int splits, bool big, hipStream_t st) { laun
 bool tn_partial_always(const GemmArgs&) { return false; }
 #endif
 
-// C[m][n] (+)= sum over splits of partial[s][m][n], in split order
+// C[m][n] (+)= sum over splits of partial[s][m][n], in split order. Workgroups past the ones that cover C add up the
+// row sums of EPI_PARTIAL_ROWSUM: rowvec[m] += sum over parts of rowsum[p][m], 32 rows per workgroup, 8 groups of lanes
+// each adding every 8th part, then the 8 sub-sums in group order (a fixed tree, like bias_grad_reduce_kernel).
+constexpr int SKR_ROWS = 32, SKR_GROUPS = 8;
 template <bool ACCUM>
 __global__ void __launch_bounds__(256)
-splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, size_t mn, int splits) {
+splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, size_t mn, int splits,
+                     floatX* __restrict__ rowvec, const float* __restrict__ rowsum, int rows, int parts, unsigned main_blocks) {
+    if (blockIdx.x >= main_blocks) {                      // workgroup-uniform
+        __shared__ float sub[SKR_GROUPS][SKR_ROWS];
+        const int rl = threadIdx.x % SKR_ROWS, grp = threadIdx.x / SKR_ROWS;
+        const int m = (int)(blockIdx.x - main_blocks) * SKR_ROWS + rl;
+        float t = 0.f;
+        if (m < rows)
+            for (int p = grp; p < parts; p += SKR_GROUPS) t += rowsum[(size_t)p * rows + m];
+        sub[grp][rl] = t;
+        __syncthreads();
+        if (grp == 0 && m < rows) {
+            float u = 0.f;
+#pragma unroll
+            for (int g2 = 0; g2 < SKR_GROUPS; g2++) u += sub[g2][rl];
+            rowvec[m] = from_f32<floatX>(to_f32(rowvec[m]) + u);
+        }
+        return;
+    }
     size_t i = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
     if (i >= mn) return;
     vecF s = ld_vec(partial + i);
@@ -700,13 +721,12 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
 #endif
                 launch_best<true, true, EPI_PARTIAL>(g, splits, big, st);
             }
-            if (dbias_in_gemm) {                                  // dbias += the splits' row sums, in split order
-                llmk::ProfScope prof("bias_grad_reduce", 0, (double)splits * parts * OC * sizeof(float), st);
-                bias_grad_reduce_kernel<<<CEIL_DIV(OC, BGR_COLS), BGR_COLS * BGR_GROUPS, 0, st>>>((floatX*)dbias, g.rowsum, OC, splits * parts);
-                LAUNCH_CHECK();
-            }
+            // dweight += the splits' partial products and, in the same launch, dbias += the row sums (in split order)
             llmk::ProfScope prof("splitk_reduce", 0, (double)mn * splits * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
-            splitk_reduce_kernel<true><<<(unsigned)CEIL_DIV(mn / 4, (size_t)256), 256, 0, st>>>((floatX*)dweight, g.partial, mn, splits);
+            const unsigned main_blocks = (unsigned)CEIL_DIV(mn / 4, (size_t)256);
+            const unsigned bias_blocks = dbias_in_gemm ? (unsigned)CEIL_DIV(OC, SKR_ROWS) : 0u;
+            splitk_reduce_kernel<true><<<main_blocks + bias_blocks, 256, 0, st>>>((floatX*)dweight, g.partial, mn, splits,
+                                                                               (floatX*)dbias, g.rowsum, OC, splits * parts, main_blocks);
             LAUNCH_CHECK();
         }
     }
