@@ -54,7 +54,7 @@ struct GemmArgs {
     const floatX* bias;   // [N] or nullptr                         (EPI_BIAS*)
     floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU)
     float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL*)
-    float* rowsum;        // [splits * ROWSUM_PARTS][M] fp32        (EPI_PARTIAL_ROWSUM)
+    float* rowsum;        // [splits * WGN][M] fp32 (WGN: column waves of the tile configuration)  (EPI_PARTIAL_ROWSUM)
     int k_per_split;      // multiple of the K block
     int splits;
 };
