@@ -503,12 +503,12 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
     const int R = m->recompute;
 
     const float dloss = 1.0f / (float)(B * T * grad_accum_steps);
+    // the clears run on the GPU while the host stages and checks the targets
+    xptr dresidual = a.scratch_btc;
+    llmk_zero(dresidual, B * T * C * X, st);
     hipCheck(hipMemcpyAsync(m->targets, targets, B * T * sizeof(int), hipMemcpyHostToDevice, st));
     token_check(targets, B * T, (int)V);
     llmk_fused_classifier(a.output, a.losses, dloss, m->targets, (int)B, (int)T, (int)V, (int)Vp, 1, st);
-
-    xptr dresidual = a.scratch_btc;
-    llmk_zero(dresidual, B * T * C * X, st);
     float* scratchF = (float*)a.output;
 
     llmk_matmul_backward(a.scratch_bt4c, g.wte, nullptr, a.output, a.lnf, p.wte, nullptr, (int)B, (int)T, (int)C, (int)Vp, st, nullptr, 1);
