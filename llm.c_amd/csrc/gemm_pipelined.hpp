@@ -470,7 +470,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
-        constexpr bool EARLY0 = EPI != EPI_ACCUM && EPI != EPI_DGELU && !IS_PARTIAL;
+        constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
         int next_kbeg = 0, next_nkb = 0;
         bool early0 = false;
         if (have_next) {
