@@ -24,7 +24,8 @@
  *     message and return instead, for tests; read it with llmk_last_error().
  *
  * Shape preconditions: C % 8 == 0 (bf16) / C % 4 == 0 (fp32) for every row length,
- * head size 64 for attention (C == 64 * NH), 16-byte aligned pointers.
+ * head size up to 128 for attention (the bf16 build's MFMA kernels cover 64, the size of every
+ * GPT-2 model; other sizes take one-wave-per-row kernels), 16-byte aligned pointers.
  */
 #ifndef LLMK_H
 #define LLMK_H

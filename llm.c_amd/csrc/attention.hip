@@ -990,101 +990,175 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
     }
 }
 
-#else
+#endif  // !LLMK_FP32
+
 // =============================================================================================
-// fp32 build: one wavefront per row, lanes = head dimensions (hs <= 64)
+// Any head size up to 128, either storage type: one wavefront per row, lane l holds head dimensions l and l + 64
+// (EPL = 2) or l alone (EPL = 1, hs <= 64). All arithmetic in fp32. The fp32 build's only path; the bf16 build takes
+// it for the head sizes its MFMA kernels do not cover (80, 96 and 128 in the GPT-3 descriptors, train_gpt2.cu:538-559).
 // =============================================================================================
+template <int EPL>
 __global__ void __launch_bounds__(256)
-att_forward_f32_kernel(float* __restrict__ out, float* __restrict__ stats, const float* __restrict__ qkv, int B, int T,
-                       int NH, int hs) {
+att_forward_rows_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int B, int T,
+                        int NH, int hs) {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);       // (b, h, t)
     if (row >= (size_t)B * NH * T) return;
     const int t = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
     const int C = NH * hs;
     const size_t C3 = 3 * (size_t)C;
-    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * hs;
     const float scale = 1.0f / sqrtf((float)hs);
-    const bool act = lane < hs;
-    const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
-    float m = -INFINITY, l = 0.f, acc = 0.f;
+    bool act[EPL];
+    float q[EPL], acc[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        act[e] = lane + 64 * e < hs;
+        q[e] = act[e] ? to_f32(base[(size_t)t * C3 + lane + 64 * e]) : 0.f;
+        acc[e] = 0.f;
+    }
+    float m = -INFINITY, l = 0.f;
     for (int t2 = 0; t2 <= t; t2++) {
-        const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
-        const float s = wave_sum(q * k) * scale;
+        float qk = 0.f, v[EPL];
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            const float k = act[e] ? to_f32(base[(size_t)t2 * C3 + C + lane + 64 * e]) : 0.f;
+            v[e] = act[e] ? to_f32(base[(size_t)t2 * C3 + 2 * C + lane + 64 * e]) : 0.f;
+            qk = e == 0 ? q[e] * k : qk + q[e] * k;
+        }
+        const float s = wave_sum(qk) * scale;
         const float m_new = fmaxf(m, s);
         const float alpha = expf(m - m_new), p = expf(s - m_new);
-        const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
-        acc = acc * alpha + p * v;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) acc[e] = acc[e] * alpha + p * v[e];
         l = l * alpha + p;
         m = m_new;
     }
-    if (act) out[((size_t)b * T + t) * C + h * hs + lane] = acc / l;
+#pragma unroll
+    for (int e = 0; e < EPL; e++)
+        if (act[e]) out[((size_t)b * T + t) * C + h * hs + lane + 64 * e] = from_f32<floatX>(acc[e] / l);
     if (stats && lane == 0) stats[((size_t)b * NH + h) * T + t] = m + logf(l);
 }
 
 // dQ: one wave per query row
+template <int EPL>
 __global__ void __launch_bounds__(256)
-att_backward_dq_f32_kernel(float* __restrict__ dqkv, const float* __restrict__ dout, const float* __restrict__ qkv,
-                           const float* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
+att_backward_dq_rows_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                            const floatX* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= (size_t)B * NH * T) return;
     const int t = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
     const int C = NH * hs;
     const size_t C3 = 3 * (size_t)C;
-    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * hs;
     const float scale = 1.0f / sqrtf((float)hs);
-    const bool act = lane < hs;
     const size_t orow = ((size_t)b * T + t) * C + h * hs;
-    const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
-    const float go = act ? dout[orow + lane] : 0.f;
-    const float dsum = wave_sum(act ? go * o[orow + lane] : 0.f);
-    const float lse = stats[((size_t)b * NH + h) * T + t];
-    float dq = 0.f;
-    for (int t2 = 0; t2 <= t; t2++) {
-        const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
-        const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
-        const float s = wave_sum(q * k) * scale;
-        const float dp = wave_sum(go * v);
-        const float p = expf(s - lse);
-        dq += p * (dp - dsum) * scale * k;
+    bool act[EPL];
+    float q[EPL], go[EPL], dq[EPL], go_o = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        const int d = lane + 64 * e;
+        act[e] = d < hs;
+        q[e] = act[e] ? to_f32(base[(size_t)t * C3 + d]) : 0.f;
+        go[e] = act[e] ? to_f32(dout[orow + d]) : 0.f;
+        const float prod = act[e] ? go[e] * to_f32(o[orow + d]) : 0.f;
+        go_o = e == 0 ? prod : go_o + prod;
+        dq[e] = 0.f;
     }
-    if (act) dqkv[((size_t)b * T + t) * C3 + h * hs + lane] = dq;
+    const float dsum = wave_sum(go_o);
+    const float lse = stats[((size_t)b * NH + h) * T + t];
+    for (int t2 = 0; t2 <= t; t2++) {
+        float k[EPL], qk = 0.f, gv = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            const int d = lane + 64 * e;
+            k[e] = act[e] ? to_f32(base[(size_t)t2 * C3 + C + d]) : 0.f;
+            const float v = act[e] ? to_f32(base[(size_t)t2 * C3 + 2 * C + d]) : 0.f;
+            qk = e == 0 ? q[e] * k[e] : qk + q[e] * k[e];
+            gv = e == 0 ? go[e] * v : gv + go[e] * v;
+        }
+        const float s = wave_sum(qk) * scale;
+        const float dp = wave_sum(gv);
+        const float p = expf(s - lse);
+#pragma unroll
+        for (int e = 0; e < EPL; e++) dq[e] += p * (dp - dsum) * scale * k[e];
+    }
+#pragma unroll
+    for (int e = 0; e < EPL; e++)
+        if (act[e]) dqkv[((size_t)b * T + t) * C3 + h * hs + lane + 64 * e] = from_f32<floatX>(dq[e]);
 }
 
 // dK, dV: one wave per key row
+template <int EPL>
 __global__ void __launch_bounds__(256)
-att_backward_dkdv_f32_kernel(float* __restrict__ dqkv, const float* __restrict__ dout, const float* __restrict__ qkv,
-                             const float* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
+att_backward_dkdv_rows_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
+                              const floatX* __restrict__ o, const float* __restrict__ stats, int B, int T, int NH, int hs) {
     const int lane = threadIdx.x & 63;
     const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (row >= (size_t)B * NH * T) return;
     const int t2 = (int)(row % T), h = (int)((row / T) % NH), b = (int)(row / ((size_t)T * NH));
     const int C = NH * hs;
     const size_t C3 = 3 * (size_t)C;
-    const float* base = qkv + (size_t)b * T * C3 + h * hs;
+    const floatX* base = qkv + (size_t)b * T * C3 + h * hs;
     const float scale = 1.0f / sqrtf((float)hs);
-    const bool act = lane < hs;
-    const float k = act ? base[(size_t)t2 * C3 + C + lane] : 0.f;
-    const float v = act ? base[(size_t)t2 * C3 + 2 * C + lane] : 0.f;
-    float dk = 0.f, dv = 0.f;
+    bool act[EPL];
+    float k[EPL], v[EPL], dk[EPL], dv[EPL];
+#pragma unroll
+    for (int e = 0; e < EPL; e++) {
+        const int d = lane + 64 * e;
+        act[e] = d < hs;
+        k[e] = act[e] ? to_f32(base[(size_t)t2 * C3 + C + d]) : 0.f;
+        v[e] = act[e] ? to_f32(base[(size_t)t2 * C3 + 2 * C + d]) : 0.f;
+        dk[e] = dv[e] = 0.f;
+    }
     for (int t = t2; t < T; t++) {
         const size_t orow = ((size_t)b * T + t) * C + h * hs;
-        const float q = act ? base[(size_t)t * C3 + lane] : 0.f;
-        const float go = act ? dout[orow + lane] : 0.f;
-        const float dsum = wave_sum(act ? go * o[orow + lane] : 0.f);
-        const float s = wave_sum(q * k) * scale;
-        const float dp = wave_sum(go * v);
+        float q[EPL], go[EPL], go_o = 0.f, qk = 0.f, gv = 0.f;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            const int d = lane + 64 * e;
+            q[e] = act[e] ? to_f32(base[(size_t)t * C3 + d]) : 0.f;
+            go[e] = act[e] ? to_f32(dout[orow + d]) : 0.f;
+            const float prod = act[e] ? go[e] * to_f32(o[orow + d]) : 0.f;
+            go_o = e == 0 ? prod : go_o + prod;
+            qk = e == 0 ? q[e] * k[e] : qk + q[e] * k[e];
+            gv = e == 0 ? go[e] * v[e] : gv + go[e] * v[e];
+        }
+        const float dsum = wave_sum(go_o);
+        const float s = wave_sum(qk) * scale;
+        const float dp = wave_sum(gv);
         const float p = expf(s - stats[((size_t)b * NH + h) * T + t]);
-        dv += p * go;
-        dk += p * (dp - dsum) * scale * q;
+#pragma unroll
+        for (int e = 0; e < EPL; e++) {
+            dv[e] += p * go[e];
+            dk[e] += p * (dp - dsum) * scale * q[e];
+        }
     }
-    if (act) {
-        dqkv[((size_t)b * T + t2) * C3 + C + h * hs + lane] = dk;
-        dqkv[((size_t)b * T + t2) * C3 + 2 * C + h * hs + lane] = dv;
+#pragma unroll
+    for (int e = 0; e < EPL; e++)
+        if (act[e]) {
+            dqkv[((size_t)b * T + t2) * C3 + C + h * hs + lane + 64 * e] = from_f32<floatX>(dk[e]);
+            dqkv[((size_t)b * T + t2) * C3 + 2 * C + h * hs + lane + 64 * e] = from_f32<floatX>(dv[e]);
+        }
+}
+
+void launch_forward_rows(floatX* out, float* stats, const floatX* qkv, int B, int T, int NH, int hs, hipStream_t st) {
+    const unsigned blocks = (unsigned)CEIL_DIV((size_t)B * NH * T, (size_t)4);
+    if (hs <= 64) att_forward_rows_kernel<1><<<blocks, 256, 0, st>>>(out, stats, qkv, B, T, NH, hs);
+    else att_forward_rows_kernel<2><<<blocks, 256, 0, st>>>(out, stats, qkv, B, T, NH, hs);
+}
+void launch_backward_rows(floatX* dqkv, const floatX* dout, const floatX* qkv, const floatX* o, const float* stats, int B,
+                          int T, int NH, int hs, hipStream_t st) {
+    const unsigned blocks = (unsigned)CEIL_DIV((size_t)B * NH * T, (size_t)4);
+    if (hs <= 64) {
+        att_backward_dq_rows_kernel<1><<<blocks, 256, 0, st>>>(dqkv, dout, qkv, o, stats, B, T, NH, hs);
+        att_backward_dkdv_rows_kernel<1><<<blocks, 256, 0, st>>>(dqkv, dout, qkv, o, stats, B, T, NH, hs);
+    } else {
+        att_backward_dq_rows_kernel<2><<<blocks, 256, 0, st>>>(dqkv, dout, qkv, o, stats, B, T, NH, hs);
+        att_backward_dkdv_rows_kernel<2><<<blocks, 256, 0, st>>>(dqkv, dout, qkv, o, stats, B, T, NH, hs);
     }
 }
-#endif
 
 }  // namespace
 
@@ -1098,18 +1172,19 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
     hipStream_t st = (hipStream_t)stream;
     const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
     llmk::ProfScope prof("attention_forward", fwd_flops, 4.0 * B * T * C * sizeof(floatX), st);
+    LLMK_REQUIRE(hs <= 128, "attention_forward: head size %d unsupported (up to 128)", hs);
 #if !defined(LLMK_FP32)
-    LLMK_REQUIRE(hs == HS, "attention_forward: head size %d unsupported (bf16 build handles 64)", hs);
-    LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
-    if (T % 64 == 0)
-        fa_forward_dma_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
-    else
-        fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
-#else
-    LLMK_REQUIRE(hs <= 64, "attention_forward: head size %d unsupported (fp32 build handles <= 64)", hs);
-    const size_t rows = (size_t)B * NH * T;
-    att_forward_f32_kernel<<<(unsigned)CEIL_DIV(rows, (size_t)4), 256, 0, st>>>((float*)out, stats, (const float*)inp, B, T, NH, hs);
+    if (hs == HS) {
+        LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
+        if (T % 64 == 0)
+            fa_forward_dma_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+        else
+            fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+        LAUNCH_CHECK();
+        return;
+    }
 #endif
+    launch_forward_rows((floatX*)out, stats, (const floatX*)inp, B, T, NH, hs, st);
     LAUNCH_CHECK();
 }
 
@@ -1121,49 +1196,47 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
     const int hs = C / NH;
     if ((size_t)B * T == 0) return;
     hipStream_t st = (hipStream_t)stream;
+    LLMK_REQUIRE(hs <= 128, "attention_backward: head size %d unsupported (up to 128)", hs);
 #if !defined(LLMK_FP32)
-    LLMK_REQUIRE(hs == HS, "attention_backward: head size %d unsupported (bf16 build handles 64)", hs);
-    float* Dsum = (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
-    const size_t nrows = (size_t)B * T * NH;
-    const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
-    const dim3 grid(CEIL_DIV(T, 128), B * NH);
-    // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x on dK/dV, 1.0x on dQ
-    if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
-        {
-            llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-            fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
-            LAUNCH_CHECK();
-        }
-        llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-        if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
-            fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-        else
-            fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-        LAUNCH_CHECK();
-    } else {
-        {
-            llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
-            fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
-            LAUNCH_CHECK();
-        }
-        {
+    if (hs == HS) {
+        float* Dsum = (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
+        const size_t nrows = (size_t)B * T * NH;
+        const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
+        const dim3 grid(CEIL_DIV(T, 128), B * NH);
+        // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x on dK/dV, 1.0x on dQ
+        if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
+            {
+                llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+                fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
+                LAUNCH_CHECK();
+            }
             llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-            fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
+                fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            else
+                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            LAUNCH_CHECK();
+        } else {
+            {
+                llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
+                fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
+                LAUNCH_CHECK();
+            }
+            {
+                llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+                LAUNCH_CHECK();
+            }
+            llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
+            fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
             LAUNCH_CHECK();
         }
-        llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
-        fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-        LAUNCH_CHECK();
+        return;
     }
-#else
-    LLMK_REQUIRE(hs <= 64, "attention_backward: head size %d unsupported (fp32 build handles <= 64)", hs);
-    const size_t rows = (size_t)B * NH * T;
-    const unsigned blocks = (unsigned)CEIL_DIV(rows, (size_t)4);
-    att_backward_dq_f32_kernel<<<blocks, 256, 0, st>>>((float*)dqkvr, (const float*)dout, (const float*)qkvr, (const float*)o, stats, B, T, NH, hs);
-    LAUNCH_CHECK();
-    att_backward_dkdv_f32_kernel<<<blocks, 256, 0, st>>>((float*)dqkvr, (const float*)dout, (const float*)qkvr, (const float*)o, stats, B, T, NH, hs);
-    LAUNCH_CHECK();
 #endif
+    llmk::ProfScope prof("attention_backward_rows", 2.5 * 4.0 * B * NH * hs * ((double)T * (T + 1) / 2), 6.0 * B * T * C * sizeof(floatX), st);
+    launch_backward_rows((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, B, T, NH, hs, st);
+    LAUNCH_CHECK();
 }
 
 }  // extern "C"

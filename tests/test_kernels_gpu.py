@@ -366,8 +366,7 @@ def test_matmul_backward_gelu(precision, fusion, M, Cc, OC):
 
 
 # ------------------------------------------------------------------------------------------------
-def attention_case(precision, B, T, NH, seed=0):
-    hs = 64
+def attention_case(precision, B, T, NH, seed=0, hs=64):
     Cc = NH * hs
     qkv = G.rounded(rnd((B, T, 3 * Cc), seed, 1.0), precision)
     g = G.rounded(rnd((B, T, Cc), seed + 1), precision)
@@ -406,6 +405,26 @@ def test_attention_forward_backward(precision, B, T, NH):
         L.llmk_attention_forward(G.ptr(d_o2), None, G.ptr(d_q2), B, T, NH, Cc, None)
         G.sync()
         assert torch.equal(d_o[:, :T // 2], d_o2[:, :T // 2])
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("hs", [32, 80, 96, 128])
+@pytest.mark.parametrize("B,T,NH", [(2, 96, 2), (1, 130, 3)])
+def test_attention_other_head_sizes(precision, hs, B, T, NH):
+    """Head sizes of the GPT-3 descriptors (train_gpt2.cu:538-559) and a small one: the one-wave-per-row kernels."""
+    L = G.lib(precision)
+    qkv, g, ro, rlse, rd, Cc = attention_case(precision, B, T, NH, seed=hs, hs=hs)
+    d_qkv, d_g = G.dev(qkv, precision), G.dev(g, precision)
+    d_o = G.dev(np.zeros((B, T, Cc), np.float32), precision)
+    d_lse = G.dev(np.zeros((B, NH, T), np.float32))
+    L.llmk_attention_forward(G.ptr(d_o), G.ptr(d_lse), G.ptr(d_qkv), B, T, NH, Cc, None)
+    close(G.host(d_o), ro, **tol(precision, 1e-5, bf16_atol=2e-2), what="out")
+    close(G.host(d_lse), rlse, rtol=1e-5, atol=1e-4, what="stats")                  # fp32 arithmetic in both builds
+    d_d = G.dev(np.full((B, T, 3 * Cc), 3.0, np.float32), precision)
+    L.llmk_attention_backward(G.ptr(d_d), G.ptr(d_g), G.ptr(d_qkv), G.ptr(d_o), G.ptr(d_lse), B, T, NH, Cc, None)
+    scale = np.abs(rd).max()
+    close(G.host(d_d), rd, **tol(precision, 1e-4 * scale, bf16_rel=1.0 / 32, bf16_atol=2e-2 * scale), what="dqkv")
     G.check_no_error(L)
 
 

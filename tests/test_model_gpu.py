@@ -137,9 +137,10 @@ def test_fp32_small_model_vs_oracle_all_modes(recompute, gelu_fusion):
     m.free()
 
 
-@pytest.mark.parametrize("heads,channels", [(16, 1024), (25, 1600)])
+@pytest.mark.parametrize("heads,channels", [(16, 1024), (25, 1600), (16, 1536), (4, 512)])
 def test_wider_gpt2_layers_vs_oracle(heads, channels):
-    # the layer widths of GPT-2 350M (d24) and 1558M (d48), two layers deep with a small vocabulary so that the
+    # the layer widths of GPT-2 350M (d24) and 1558M (d48), and of GPT-3's 760M descriptor (head size 96,
+    # train_gpt2.cu:538-559) plus a narrow model with head size 128, two layers deep with a small vocabulary so that the
     # CPU oracle finishes in seconds: fp32 to the fp32 bar, bf16 to the bf16 bar. The learning rate keeps the loss of
     # this one repeated batch of order 1 over the ten steps, where a relative bound on it means something
     cfg = ol.Config(64, 2000, 2048, 2, heads, channels)
