@@ -110,6 +110,9 @@ def test_dataloader_without_shuffle_is_a_strided_walk(L, tmp_path):
     n = B * T
     ld = Loader(L, pattern, B, T, rank, nproc, 0)
     assert L.dataloader_num_shards(ld.h) == 3 and L.dataloader_num_tokens(ld.h) == sum(SHARD_SIZES)
+    assert L.dataloader_should_shuffle(ld.h) == 0
+    # samples of the current shard for this process group: (tokens - 1) // (processes * B * T), llmc/dataloader.h:96
+    assert L.dataloader_shard_num_samples(ld.h) == (toks[0].size - 1) // (nproc * n)
     for epoch in range(2):
         for s, t in enumerate(toks):
             for k in range((t.size - 1) // (nproc * n)):
@@ -257,6 +260,21 @@ def test_evalloader_layout_and_scoring(L, tmp_path):
                 means.append(np.float32(losses[i].reshape(B, T)[row][want_mask == 1].astype(np.float64).mean()))
             want_correct += int(np.argmin(means)) == lab
         assert correct[i] == want_correct
+    # evalloader_reset (llmc/dataloader.h:298) goes back to the process's first example: the first batch comes again
+    h = L.evalloader_create()
+    L.evalloader_init(h, path.encode(), B, T, 0, 1)
+    L.evalloader_next_batch(h); L.evalloader_next_batch(h)
+    assert L.evalloader_current_example_index(h) == 4
+    L.evalloader_reset(h)
+    assert L.evalloader_current_example_index(h) == 0
+    L.evalloader_next_batch(h)
+    again = np.ctypeslib.as_array(L.evalloader_inputs(h), shape=(B * T,)).reshape(B, T)
+    np.testing.assert_array_equal(np.frombuffer(C.string_at(L.evalloader_mask(h), B * T), np.int8), mask[0])
+    for slot in range(2):                                          # the tokens past a row's end are left as they were
+        lab, ctx, comps = examples[slot]
+        for c, comp in enumerate(comps):
+            np.testing.assert_array_equal(again[slot * 4 + c][:len(ctx) + len(comp)], ctx + comp)
+    L.evalloader_free(h)
 
 
 # ---- learning-rate schedules -------------------------------------------------------------------------------------

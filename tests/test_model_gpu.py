@@ -462,3 +462,57 @@ def test_bf16_full_size_step_properties():
     wte = m.params()[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels)
     assert (wte[cfg.vocab_size:] == 0).all()
     m.free()
+
+
+@pytest.mark.parametrize("descriptor,expect", [("d12", (1024, 50257, 50304, 12, 12, 768)),
+                                               ("d24", (1024, 50257, 50304, 24, 16, 1024)),
+                                               ("gpt3:c384", (2048, 50257, 50304, 6, 6, 384)),
+                                               ("gpt3:c768", (2048, 50257, 50304, 12, 12, 768))])
+def test_descriptors_give_the_reference_shapes(descriptor, expect):
+    """Model descriptors (train_gpt2.cu:511-570): hyperparameters, the sixteen tensor sizes and the parameter count."""
+    L = G.lib("bf16")
+    h = L.gpt2_create()
+    L.gpt2_build_from_descriptor(h, descriptor.encode())
+    six = (C.c_int * 6)()
+    L.gpt2_get_config(h, six)
+    assert tuple(six) == expect
+    sizes = (C.c_size_t * 16)()
+    L.gpt2_param_sizes(h, sizes)
+    ref_sizes, total = ol.param_sizes(ol.Config(*expect))
+    assert list(sizes) == ref_sizes
+    assert L.gpt2_num_parameters(h) == total
+    L.gpt2_free(h)
+
+
+def test_accessors_rng_state_and_event_profile():
+    """What a caller outside the step uses: device properties, the activation footprint, the stochastic-rounding
+    counter that checkpoints carry (train_gpt2.cu:1225,1275), and the per-family event profile."""
+    L = G.lib("bf16")
+    ncu, thr, name = C.c_int(0), C.c_int(0), C.create_string_buffer(256)
+    L.llmk_device_props(C.byref(ncu), C.byref(thr), name)
+    assert ncu.value >= 8 and ncu.value % 8 == 0 and thr.value >= 1024 and len(name.value) > 0
+    cfg = ol.Config(64, 128, 128, 2, 2, 128)
+    B, T = 2, 64
+    m = Model("bf16", cfg, B, T, seed=5, recompute=0)
+    small = L.gpt2_activation_bytes(m.h)
+    assert small > 2 * B * T * cfg.padded_vocab_size                       # at least the bf16 logits
+    L.gpt2_set_rng_state(m.h, 0x123456789ABCDEF)
+    assert L.gpt2_get_rng_state(m.h) == 0x123456789ABCDEF
+    inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 3)
+    L.llmk_profile_reset()
+    L.llmk_profile_enable(1)
+    m.step(inp, tgt, 1, 1e-3, 0.9, 0.95, 1e-8, 0.0)
+    L.llmk_profile_enable(0)
+    assert L.gpt2_get_rng_state(m.h) != 0x123456789ABCDEF                   # the update drew rounding seeds
+    fams = {}
+    for i in range(L.llmk_profile_count()):
+        nm, calls, ms, fl, by = C.create_string_buffer(64), C.c_int(0), C.c_double(0), C.c_double(0), C.c_double(0)
+        L.llmk_profile_get(i, nm, C.byref(calls), C.byref(ms), C.byref(fl), C.byref(by))
+        fams[nm.value.decode()] = (calls.value, ms.value, fl.value, by.value)
+    for need in ("attention_forward", "fused_classifier", "adamw_update", "layernorm_backward", "encoder_forward"):
+        assert need in fams and fams[need][0] >= 1 and fams[need][1] > 0.0, (need, sorted(fams))
+    assert fams["adamw_update"][0] == 16 and fams["attention_forward"][0] == cfg.num_layers
+    assert fams["attention_forward"][2] == pytest.approx(4.0 * B * cfg.num_heads * 64 * (T * (T + 1) / 2) * cfg.num_layers)
+    L.llmk_profile_reset()
+    assert L.llmk_profile_count() == 0
+    m.free()
