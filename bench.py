@@ -29,8 +29,8 @@ METRIC = "train tokens/sec + MFU, GPT-2 124M bf16 B=64 T=1024, 1 MI355X"
 # the counters read for a copy kernel of known size (profiles/train_step_gpt2_124M_b64_t1024_hbm_traffic.txt has the
 # commands and the table). Valid for the default workload only. FETCH_SIZE counts L2 fills whether the Infinity Cache
 # or HBM served them.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemm_nn": 967529981, "gemm_nn_dgelu": 1373351060, "gemm_tn_splitk": 869401086,
-                                     "gemm_nt": 964177709, "gemm_nt_gelu": 1243561247}
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemm_nn": 933442355, "gemm_nn_dgelu": 1439589990, "gemm_tn_splitk": 824298433,
+                                     "gemm_nt": 888288405, "gemm_nt_gelu": 1286917324}
 
 # kernel families timed by the library -> roofline that bounds them
 MFMA_BOUND = {"gemm_nt", "gemm_nt_gelu", "gemm_nn", "gemm_nn_dgelu", "gemm_tn", "gemm_tn_splitk",
