@@ -53,7 +53,8 @@ int dataloader_should_shuffle(const LLMK_DataLoader* loader);
  * generator (llmc/rand.h:98-104: 8 bytes that the reference leaves unset and this library writes as zero, left_,
  * next_, 624 state words, MATRIX_A). Returns the byte count; buf may be NULL to ask for it. 0 without shuffling. */
 size_t dataloader_get_shuffle_state(const LLMK_DataLoader* loader, void* buf);
-/* ... and as load_state reads it back (train_gpt2.cu:1289-1308); follow with dataloader_resume. Returns bytes consumed. */
+/* ... and as load_state reads it back (train_gpt2.cu:1289-1308); follow with dataloader_resume. Returns bytes consumed.
+ * bytes == 0 is the state of a loader that does not shuffle: the loader stops shuffling (train_gpt2.cu:1289). */
 size_t dataloader_set_shuffle_state(LLMK_DataLoader* loader, const void* buf, size_t bytes);
 
 /* ---- multiple-choice evaluation file, e.g. HellaSwag (llmc/dataloader.h:250-518) ---------------

@@ -572,8 +572,9 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
     g.lda = C; g.ldb = C; g.ldc = OC; g.bias = (const floatX*)bias; g.k_per_split = CEIL_DIV(C, K_STEP) * K_STEP;
     const int num_cu = llmk::device_info().num_cu;
     const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(OC, BIG_TILE) >= (size_t)num_cu;
-    llmk::ProfScope prof((pre_gelu && gelu_fusion >= 1) ? "gemm_nt_gelu" : "gemm_nt", 2.0 * M * (double)OC * C,
-                         ((double)M * C + (double)OC * C + (double)M * OC) * sizeof(floatX), st);
+    const bool gelu_in_gemm = pre_gelu && gelu_fusion >= 1;            // then the kernel writes two (M, OC) tensors
+    llmk::ProfScope prof(gelu_in_gemm ? "gemm_nt_gelu" : "gemm_nt", 2.0 * M * (double)OC * C,
+                         ((double)M * C + (double)OC * C + (gelu_in_gemm ? 2.0 : 1.0) * M * OC) * sizeof(floatX), st);
     if (pre_gelu && gelu_fusion >= 1) {
         g.C = (floatX*)out; g.aux = (floatX*)pre_gelu;
         launch_best<false, false, EPI_BIAS_GELU>(g, 1, big, st);
@@ -657,8 +658,9 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         const bool fused = pre_gelu && gelu_fusion >= 2 && big && aligned16(pre_gelu) && pipelined_ok(g);
 #endif
         {
+            // with GELU backward in the epilogue the kernel also reads the (M, C) pre-activations
             llmk::ProfScope prof(fused ? "gemm_nn_dgelu" : "gemm_nn", 2.0 * M * (double)OC * C,
-                                 ((double)M * OC + (double)OC * C + (double)M * C) * sizeof(floatX), st);
+                                 ((double)M * OC + (double)OC * C + (fused ? 2.0 : 1.0) * M * C) * sizeof(floatX), st);
             if (fused) {
                 g.aux = (floatX*)pre_gelu;
 #if defined(LLMK_FP32)

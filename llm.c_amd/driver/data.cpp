@@ -252,6 +252,7 @@ size_t dataloader_get_shuffle_state(const LLMK_DataLoader* l, void* buf) {
 }
 
 size_t dataloader_set_shuffle_state(LLMK_DataLoader* l, const void* buf, size_t bytes) {
+    if (bytes == 0) { l->should_shuffle = false; return 0; }      // the state of a loader that does not shuffle
     const char* p = (const char*)buf;
     const char* end = p + bytes;
     auto get = [&](void* dst, size_t n) {

@@ -130,7 +130,28 @@ void* malloc_and_point_parameters(ParameterTensors* p, const size_t* elems, size
     return mem;
 }
 
+// What the kernels behind this driver can run, checked before anything is allocated: channels a multiple of 8 (one
+// 16-byte vector of bf16), at most 64 lanes x 8 vectors per row in LayerNorm backward (4096 channels in bf16, 2048 in
+// fp32), heads of at most 128 channels.
+static void check_config(const LLMK_GPT2* m) {
+    const GPT2Config& c = m->config;
+    const int max_channels = 8 * 64 * (16 / (int)m->X);
+    const char* why = nullptr;
+    if (c.channels <= 0 || c.num_heads <= 0 || c.num_layers <= 0 || c.max_seq_len <= 0) why = "sizes must be positive";
+    else if (c.channels % 8 != 0) why = "channels must be a multiple of 8";
+    else if (c.channels > max_channels) why = "too many channels for this precision's LayerNorm backward";
+    else if (c.channels % c.num_heads != 0) why = "channels must divide into the heads";
+    else if (c.channels / c.num_heads > 128) why = "head size above 128";
+    else if (c.padded_vocab_size < c.vocab_size || c.padded_vocab_size % 8 != 0) why = "padded vocabulary must cover the vocabulary and be a multiple of 8";
+    if (why) {
+        fprintf(stderr, "Unsupported model (layers %d, heads %d, channels %d, vocabulary %d/%d) in the %s build: %s (channels <= %d)\n",
+                c.num_layers, c.num_heads, c.channels, c.vocab_size, c.padded_vocab_size, m->X == 2 ? "bf16" : "fp32", why, max_channels);
+        exit(EXIT_FAILURE);
+    }
+}
+
 void gpt2_allocate_weights(LLMK_GPT2* m) {   // train_gpt2.cu:353
+    check_config(m);
     fill_in_parameter_sizes(m->param_elements, m->config);
     m->num_parameters = 0;
     for (int i = 0; i < NUM_PARAMETER_TENSORS; i++) m->num_parameters += m->param_elements[i];
@@ -697,9 +718,15 @@ void gpt2_load_state_with_loader(int* step, LLMK_GPT2* m, LLMK_DataLoader* loade
         // re-derive the low-precision weights from the master copy with the RNG state of the last update
         m->rng_state = m->rng_state_last_update;
         gpt2_update(m, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0.0f, 0, 1);
+    } else if (use_master == 1) {
+        // the file carries a master copy this run does not keep (train_gpt2.cu:1268-1270 warns and goes on): step over it,
+        // so that what follows is read as what it is
+        fprintf(stderr, "Warning: Master weights are present in state, but not enabled for current run.");
+        fseek(f, (long)(m->num_parameters * sizeof(float)), SEEK_CUR);
     }
     m->rng_state = final_rng;
     if (loader) {
+        if (hdr[5] != 1) dataloader_set_shuffle_state(loader, nullptr, 0);     // the loader takes the file's flag (train_gpt2.cu:1289)
         if (hdr[5] == 1) {
             const long at = ftell(f);
             fseek(f, 0, SEEK_END);

@@ -177,7 +177,9 @@ int main(int argc, char** argv) {
     const bool resuming_run = resume_max_step != -1;
     LLMK_GPT2* model = gpt2_create();
     gpt2_set_options(model, use_master_weights, recompute, gelu_fusion);
-    if (resuming_run) gpt2_build_from_checkpoint(model, resume_model.c_str(), /*weight_init*/ 0);
+    // with master weights the parameters are re-derived from the state file; without them they are in the model file only
+    // (train_gpt2.cu:1577-1578)
+    if (resuming_run) gpt2_build_from_checkpoint(model, resume_model.c_str(), /*weight_init*/ use_master_weights ? 0 : 1);
     else if (ends_with(load_filename, ".bin")) gpt2_build_from_checkpoint(model, load_filename, 1);
     else gpt2_build_from_descriptor(model, load_filename);
     int cfg[6];

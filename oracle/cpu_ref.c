@@ -17,11 +17,14 @@
  *                             closed forms (constant rows, T=1 attention, uniform logits,
  *                             AdamW first step) and central finite differences
  *   whole model               the compiled reference on a tiny GPT-2 (golden fixture committed)
- *   mixed-precision AdamW,    no CPU counterpart exists in the reference (CUDA only): pinned by
- *   stochastic rounding       closed forms/invariants (rounding is to one of the two bf16
- *                             neighbours, unbiased in expectation, SquirrelNoise5 constants
- *                             against llmc/cuda_utils.cuh:238-262 by hand-computed values)
- *                             => "parity unpinned" against executed reference code.
+ *   mixed-precision AdamW,    device code only in the reference (llmc/adamw.cuh, llmc/cuda_utils.cuh:238-278), so
+ *   stochastic rounding       pinned by what fixes them without the reference running
+ *                             (tests/test_oracle_optimizer_pins.py): SquirrelNoise5 by known answers worked through
+ *                             by hand from the published constants, its inverse, injectivity and avalanche; the
+ *                             noise word of an element by a walk over the reference's launch grid; the update by
+ *                             bit-equality of its fp32 state with the fp32 update (itself held to train_gpt2.c's
+ *                             AdamW over several steps) and of its bf16 parameter with the stochastic rounding of
+ *                             that state; the rounding by its exact up-probability low16/65536.
  */
 #include <math.h>
 #include <stdint.h>
