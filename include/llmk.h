@@ -149,6 +149,15 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                              int B, int T, int NH, int C, void* stream);
 
+/* The same operation for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The rowsum(dO*O) vector lives in a
+ * 4 MiB array that is part of the library's code object on every GPU instead of the grow-only workspace, so the call
+ * makes no hipMalloc/hipFree and creates no events (it is not timed by llmk_profile_*). Limit: B*NH*T <= 1048576
+ * (larger sizes are rejected with an error; GPT-2 124M at B=64, T=1024 needs 786432). Results are bit-identical to
+ * llmk_attention_backward. All calls on one GPU share the one array: calls that overlap on a GPU (two streams) race. */
+void llmk_attention_backward_static(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
+                                    int B, int T, int NH, int C, void* stream);
+
 /* ---- gelu (llmc/gelu.cuh) ----------------------------------------------------------------- */
 
 /* gelu_forward, llmc/gelu.cuh:50 */

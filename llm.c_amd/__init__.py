@@ -59,6 +59,7 @@ KERNEL_ABI = {
     "llmk_gelu_backward_bias": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "llmk_attention_forward": (None, [vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_attention_backward": (None, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "llmk_attention_backward_static": (None, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_gelu_forward": (None, [vp, vp, i32, vp]),
     "llmk_gelu_backward_inplace": (None, [vp, vp, i32, vp]),
     "llmk_fused_classifier": (None, [vp, vp, f32, vp, i32, i32, i32, i32, i32, vp]),

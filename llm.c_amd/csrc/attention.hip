@@ -1160,7 +1160,91 @@ void launch_backward_rows(floatX* dqkv, const floatX* dout, const floatX* qkv, c
     }
 }
 
+
+// ---- scratch that needs no allocation ------------------------------------------------------------------------------
+// Device memory that exists from the moment the code object is loaded: the rowsum(dO*O) vector of
+// llmk_attention_backward_static. Each GPU holds its own copy at its own address; in host code the array's name is
+// only a handle for hipGetSymbolAddress, never an address to hand to a kernel.
+constexpr size_t STATIC_SCRATCH_FLOATS = (size_t)1 << 20;        // 4 MiB: B*NH*T up to 1048576 (GPT-2 124M at B=64, T=1024 needs 786432)
+static __device__ __align__(256) float scratch[STATIC_SCRATCH_FLOATS];
+constexpr int MAX_DEVICES = 64;
+float* g_static_scratch[MAX_DEVICES];                             // per device, filled by static_scratch_setup()
+
+float* static_scratch_setup() {
+    int dev = -1;
+    HIP_CHECK(hipGetDevice(&dev));
+    if (dev < 0 || dev >= MAX_DEVICES) { llmk::fail(__FILE__, __LINE__, "device index %d out of range", dev); return nullptr; }
+    if (!g_static_scratch[dev]) {
+        void* p = nullptr;
+        hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) {
+            llmk::fail(__FILE__, __LINE__, "hipGetSymbolAddress(scratch) on device %d: %s", dev, hipGetErrorString(e));
+            return nullptr;
+        }
+        g_static_scratch[dev] = (float*)p;
+    }
+    return g_static_scratch[dev];
+}
+float* static_scratch_ptr() { return static_scratch_setup(); }    // the current device's copy (looked up once per device)
+
+// Dsum_static: device memory for the B*NH*T floats of rowsum(dO*O), or nullptr to take them from the library workspace
+// (which may allocate). With Dsum_static nothing on this path allocates: no workspace, no timing events.
+void attention_backward_impl(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
+                             int B, int T, int NH, int C, void* stream, float* Dsum_static) {
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(NH > 0 && C % NH == 0, "attention_backward: C=%d not divisible by NH=%d", C, NH);
+    LLMK_REQUIRE(stats != nullptr, "attention_backward: stats from the forward pass are required");
+    const int hs = C / NH;
+    if ((size_t)B * T == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+    LLMK_REQUIRE(hs <= 128, "attention_backward: head size %d unsupported (up to 128)", hs);
+#if !defined(LLMK_FP32)
+    if (hs == HS) {
+        float* Dsum = Dsum_static ? Dsum_static : (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
+        const size_t nrows = (size_t)B * T * NH;
+        const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
+        const dim3 grid(CEIL_DIV(T, 128), B * NH);
+        // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x on dK/dV, 1.0x on dQ
+        if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
+            {
+                llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+                fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
+                LAUNCH_CHECK();
+            }
+            llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+            if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
+                fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            else
+                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            LAUNCH_CHECK();
+        } else {
+            {
+                llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
+                fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
+                LAUNCH_CHECK();
+            }
+            {
+                llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
+                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+                LAUNCH_CHECK();
+            }
+            llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
+            fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            LAUNCH_CHECK();
+        }
+        return;
+    }
+#endif
+    llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_rows", 2.5 * 4.0 * B * NH * hs * ((double)T * (T + 1) / 2), 6.0 * B * T * C * sizeof(floatX), st);
+    launch_backward_rows((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, B, T, NH, hs, st);
+    LAUNCH_CHECK();
+}
+
 }  // namespace
+
+namespace llmk {
+void attention_static_scratch_init() { (void)static_scratch_setup(); }
+}  // namespace llmk
 
 extern "C" {
 
@@ -1190,53 +1274,18 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 
 void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                              int B, int T, int NH, int C, void* stream) {
+    attention_backward_impl(dqkvr, dout, qkvr, o, stats, B, T, NH, C, stream, nullptr);
+}
+
+void llmk_attention_backward_static(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
+                                    int B, int T, int NH, int C, void* stream) {
     if (llmk::failed()) return;
-    LLMK_REQUIRE(NH > 0 && C % NH == 0, "attention_backward: C=%d not divisible by NH=%d", C, NH);
-    LLMK_REQUIRE(stats != nullptr, "attention_backward: stats from the forward pass are required");
-    const int hs = C / NH;
-    if ((size_t)B * T == 0) return;
-    hipStream_t st = (hipStream_t)stream;
-    LLMK_REQUIRE(hs <= 128, "attention_backward: head size %d unsupported (up to 128)", hs);
-#if !defined(LLMK_FP32)
-    if (hs == HS) {
-        float* Dsum = (float*)llmk::workspace((size_t)B * NH * T * sizeof(float));
-        const size_t nrows = (size_t)B * T * NH;
-        const double fwd_flops = 4.0 * B * NH * hs * ((double)T * (T + 1) / 2);
-        const dim3 grid(CEIL_DIV(T, 128), B * NH);
-        // algorithmic backward work is 2.5x forward (5 contractions vs 2); booked 1.5x on dK/dV, 1.0x on dQ
-        if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
-            {
-                llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-                fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
-                LAUNCH_CHECK();
-            }
-            llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-            if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
-                fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-            else
-                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-            LAUNCH_CHECK();
-        } else {
-            {
-                llmk::ProfScope prof("attention_backward_dot", 0, 2.0 * B * T * C * sizeof(floatX), st);
-                fa_dot_do_o_kernel<<<(unsigned)CEIL_DIV(nrows * 8, (size_t)256), 256, 0, st>>>(Dsum, (const floatX*)dout, (const floatX*)o, B, T, NH);
-                LAUNCH_CHECK();
-            }
-            {
-                llmk::ProfScope prof("attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-                fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-                LAUNCH_CHECK();
-            }
-            llmk::ProfScope prof("attention_backward_dq", 1.0 * fwd_flops, 5.0 * B * T * C * sizeof(floatX), st);
-            fa_backward_dq_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
-            LAUNCH_CHECK();
-        }
-        return;
-    }
-#endif
-    llmk::ProfScope prof("attention_backward_rows", 2.5 * 4.0 * B * NH * hs * ((double)T * (T + 1) / 2), 6.0 * B * T * C * sizeof(floatX), st);
-    launch_backward_rows((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, B, T, NH, hs, st);
-    LAUNCH_CHECK();
+    LLMK_REQUIRE((size_t)B * (size_t)max(NH, 0) * (size_t)T <= STATIC_SCRATCH_FLOATS,
+                 "attention_backward_static: B*NH*T = %zu exceeds the %zu floats of static scratch; use llmk_attention_backward",
+                 (size_t)B * NH * T, STATIC_SCRATCH_FLOATS);
+    float* ptr = static_scratch_ptr();
+    if (!ptr) return;                                            // the failure is recorded
+    attention_backward_impl(dqkvr, dout, qkvr, o, stats, B, T, NH, C, stream, ptr);
 }
 
 }  // extern "C"

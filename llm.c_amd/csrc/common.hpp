@@ -56,6 +56,10 @@ struct ProfScope {
     ProfScope(const char* name, double flops, double bytes, hipStream_t s) : st(s), on(profiling(name)) {
         if (on) prof_begin(name, flops, bytes, st);
     }
+    // never_time: for callers that must not create events (entry points that allocate nothing)
+    ProfScope(bool never_time, const char* name, double flops, double bytes, hipStream_t s) : st(s), on(!never_time && profiling(name)) {
+        if (on) prof_begin(name, flops, bytes, st);
+    }
     ~ProfScope() { if (on) prof_end(st); }
 };
 }  // namespace llmk

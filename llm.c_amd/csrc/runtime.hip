@@ -12,6 +12,8 @@
 
 namespace llmk {
 
+void attention_static_scratch_init();     // csrc/attention.hip
+
 static DeviceInfo g_dev;
 static int g_error_mode = 0;  // 0: print + exit, 1: record
 static std::string g_last_error;
@@ -137,6 +139,7 @@ void llmk_init(int device) {
     HIP_CHECK(hipSetDevice(device));
     llmk::g_dev.ready = false;
     (void)llmk::device_info();
+    llmk::attention_static_scratch_init();       // this device's address of the attention backward's static scratch
 }
 
 void llmk_shutdown(void) {
