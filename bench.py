@@ -2,7 +2,8 @@
 """Throughput of the GPT-2 124M training step (bf16, B=64, T=1024) on one MI355X through the C ABI,
 with the reference's CPU trainer timed beside it.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-kernel-events]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-kernel-events] [--no-mfma-probe]
+                    [--no-other-configs] [--model d12|d24|d48 --batch B --recompute R]
 
 A step = gpt2_forward + gpt2_backward_and_reduce + gpt2_calculate_grad_norm (clip at 1.0) + gpt2_update
 on one batch of synthetic tokens, exactly the work of one iteration of the reference's training loop
@@ -24,13 +25,36 @@ PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA, vendor figure
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 METRIC = "train tokens/sec + MFU, GPT-2 124M bf16 B=64 T=1024, 1 MI355X"
 
-# Bytes per launch (read + written, averaged over the launches of a step) that the GEMM families move between L2 and
-# the memory side, from two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) over this same workload, scaled by what
-# the counters read for a copy kernel of known size (profiles/train_step_gpt2_124M_b64_t1024_hbm_traffic.txt has the
-# commands and the table). Valid for the default workload only. FETCH_SIZE counts L2 fills whether the Infinity Cache
-# or HBM served them.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = {"gemm_nn": 933442355, "gemm_nn_dgelu": 1439589990, "gemm_tn_splitk": 824298433,
-                                     "gemm_nt": 888288405, "gemm_nt_gelu": 1286917324}
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "train_step_gpt2_124M_b64_t1024_hbm_traffic.txt")
+KERNEL_SOURCES = ("gemm.hip", "gemm_pipelined.hpp", "common.hpp", "gelu.hpp")
+
+
+def kernel_sources_sha16():
+    """Fingerprint of the sources of the kernels whose memory traffic the profile summary records."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES:
+        with open(os.path.join(ROOT, "llm.c_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(family):
+    """Bytes per launch (read + written, averaged over the launches of a step) that a GEMM family moves between L2 and
+    the memory side: from the two rocprofv3 --pmc passes (FETCH_SIZE, WRITE_SIZE) summarised in TRAFFIC_PROFILE, scaled
+    there by what the counters read for a copy kernel of known size. The summary carries the fingerprint of the kernel
+    sources it was measured on; when the sources have changed since, the figure is stale and None is returned.
+    FETCH_SIZE counts L2 fills whether the Infinity Cache or HBM served them."""
+    try:
+        lines = open(TRAFFIC_PROFILE).read().splitlines()
+    except OSError:
+        return None
+    sha = [l.split(":", 1)[1].strip() for l in lines if l.startswith("kernel_sources_sha16:")]
+    table = [l.split(":", 1)[1].strip() for l in lines if l.startswith("family_traffic_bytes_per_launch:")]
+    if not sha or not table or sha[0] != kernel_sources_sha16():
+        return None
+    return json.loads(table[0]).get(family)
+
 
 # kernel families timed by the library -> roofline that bounds them
 MFMA_BOUND = {"gemm_nt", "gemm_nt_gelu", "gemm_nn", "gemm_nn_dgelu", "gemm_tn", "gemm_tn_splitk",
@@ -83,43 +107,60 @@ def cpu_baseline(budget_s=14.0):
                       f"OpenMP threads={cores}"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--batch", type=int, default=64)
-    ap.add_argument("--seq", type=int, default=1024)
-    ap.add_argument("--model", default="d12")
-    ap.add_argument("--recompute", type=int, default=0)   # the reference's 124M recipe runs with -r 0 (scripts/run_gpt2_124M.sh)
-    ap.add_argument("--gelu-fusion", type=int, default=2)
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-kernel-events", action="store_true")
-    ap.add_argument("--calibrate-copy", action="store_true",
-                    help="first launch one copy kernel of known size (128 MiB read, 256 MiB written): the yardstick for "
-                         "scaling FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
-    args = ap.parse_args()
-    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: this build runs the training step on ONE GPU only (no collectives are part of it); "
-              "use --gpus 1", file=sys.stderr)
-        sys.exit(2)
+class SclkSampler:
+    """Samples the driver's current shader clock (the line marked * in /sys/class/drm/card*/device/pp_dpm_sclk, in MHz) from
+    a background thread while the body of the with-statement runs; readings at or below the lowest power state are dropped."""
 
-    # the native driver and the reference's CPU trainer print their model headers with printf: send everything
-    # written to file descriptor 1 to stderr until the result line, so stdout carries exactly one JSON line
-    sys.stdout.flush()
-    real_stdout = os.dup(1)
-    os.dup2(2, 1)
+    def __init__(self, period_s=0.01):
+        import glob
+        paths = sorted(glob.glob("/sys/class/drm/card*/device/pp_dpm_sclk"))
+        self.path = paths[0] if paths else None
+        self.period = period_s
+        self.samples = []
+        self._stop = False
+        self._thread = None
 
-    import torch
-    assert torch.cuda.is_available(), "bench.py needs a GPU"
-    pkg = package()
-    L = pkg.load("bf16")           # raises if the HIP library is not built: there is no other path
-    L.llmk_init(0)
-    B, T = args.batch, args.seq
-    default_workload = (B, T, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 2)
+    def _run(self):
+        import re
+        while not self._stop:
+            try:
+                for line in open(self.path):
+                    if line.rstrip().endswith("*"):
+                        m = re.search(r"(\d+)\s*Mhz", line)
+                        if m:
+                            self.samples.append(int(m.group(1)))
+            except OSError:
+                return
+            time.sleep(self.period)
+
+    def __enter__(self):
+        if self.path:
+            import threading
+            self._thread = threading.Thread(target=self._run, daemon=True)
+            self._thread.start()
+        return self
+
+    def __exit__(self, *exc):
+        self._stop = True
+        if self._thread:
+            self._thread.join()
+        return False
+
+    def median(self):
+        busy = [s for s in self.samples if s > 600]
+        return float(np.median(busy)) if busy else None
+
+
+def default_headline(args):
+    return (args.batch, args.seq, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 2)
+
+
+def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, kernel_events, lr=6e-4):
+    """Builds the model, runs warmup + steps training steps on one synthetic batch, returns the result fields."""
+    default_workload = (B, T, model, recompute, gelu_fusion) == (64, 1024, "d12", 0, 2)
     h = L.gpt2_create()
-    L.gpt2_set_options(h, 1, args.recompute, args.gelu_fusion)
-    L.gpt2_build_from_descriptor(h, args.model.encode())
+    L.gpt2_set_options(h, 1, recompute, gelu_fusion)
+    L.gpt2_build_from_descriptor(h, model.encode())
     L.gpt2_allocate_state(h, B, T)
     cfg = (C.c_int * 6)()
     L.gpt2_get_config(h, cfg)
@@ -130,21 +171,13 @@ def main():
     inp, tgt = np.ascontiguousarray(stream[:-1]), np.ascontiguousarray(stream[1:])
     ip, tp = inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p)
 
-    if args.calibrate_copy:
-        n = 64 * 1024 * 1024
-        src = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
-        dst = torch.empty(n, dtype=torch.float32, device="cuda")
-        L.llmk_copy_and_cast_to_f32(dst.data_ptr(), src.data_ptr(), n, 0, 0, 1, None)
-        torch.cuda.synchronize()
-        del src, dst
-
     def step(t):
         L.gpt2_forward(h, ip, B, T)
         L.gpt2_backward_and_reduce(h, ip, tp, 1, 0)
         loss = L.gpt2_mean_loss(h)
         norm = L.gpt2_calculate_grad_norm(h)
         scale = 1.0 / norm if norm > 1.0 else 1.0
-        L.gpt2_update(h, 6e-4, 0.9, 0.95, 1e-8, 0.1, scale, t, 0)
+        L.gpt2_update(h, lr, 0.9, 0.95, 1e-8, 0.1, scale, t, 0)
         return loss, norm
 
     def read_profile(nsteps):
@@ -172,8 +205,8 @@ def main():
     # ~400 launches of a step costs about 1.7 % of the step; one family costs about 0.2 %).
     losses = []
     kernels = []
-    for w in range(args.warmup):
-        last = (w == args.warmup - 1) and not args.no_kernel_events
+    for w in range(warmup):
+        last = (w == warmup - 1) and kernel_events
         if last:
             torch.cuda.synchronize()
             L.llmk_profile_reset()
@@ -186,49 +219,133 @@ def main():
             kernels = read_profile(1)
     torch.cuda.synchronize()
     dominant = kernels[0]["kernel"] if kernels else None
-    if not args.no_kernel_events:
+    if kernel_events:
         L.llmk_profile_reset()
         L.llmk_profile_only(dominant.encode() if dominant else None)   # without a warmup step: every family
         L.llmk_profile_enable(1)
     t0 = time.perf_counter()
-    for s in range(args.steps):
-        losses.append(step(args.warmup + s + 1)[0])
+    for s in range(steps):
+        losses.append(step(warmup + s + 1)[0])
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     L.llmk_profile_enable(0)
 
-    ms_per_step = dt / args.steps * 1e3
-    tokens_per_s = B * T * args.steps / dt
-    mfu = L.gpt2_estimate_mfu(h, B * T, ctypes_float(dt / args.steps))
+    ms_per_step = dt / steps * 1e3
+    tokens_per_s = B * T * steps / dt
+    mfu = L.gpt2_estimate_mfu(h, B * T, C.c_float(dt / steps))
 
     roofline = None
-    if not args.no_kernel_events:
-        timed = read_profile(args.steps)
+    if kernel_events:
+        timed = read_profile(steps)
         if not kernels:
             kernels = timed
         d = timed[0]                           # the dominant family, timed live inside the timed steps
         roofline = {"kernel": d["kernel"], "bound": d["bound"], "achieved": d["achieved"], "peak": d["peak"],
                     "unit": d["unit"], "frac": d["frac"],
-                    "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH.get(d["kernel"]) if default_workload else None,
+                    "traffic": measured_traffic(d["kernel"]) if default_workload else None,
                     "algorithmic_bytes_per_launch": d["bytes_per_launch"],
                     "avg_launch_ms": d["avg_launch_ms"], "launches_per_step": d["launches_per_step"],
                     "ms_per_step": d["ms_per_step"]}
+        L.llmk_profile_reset()
+        L.llmk_profile_only(None)
     L.gpt2_free(h)
-
-    out = {
-        "metric": METRIC, "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+    return {
+        "value": tokens_per_s, "unit": "tokens/s", "n_gpus": 1, "steps": steps,
+        "warmup": warmup, "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": {"workload": f"GPT-2 {args.model} ({nparams} params) full train step, bf16 + fp32 master weights/AdamW, "
+        "config": {"workload": f"GPT-2 {model} ({nparams} params) full train step, bf16 + fp32 master weights/AdamW, "
                                f"flash attention, clip 1.0" +
                                {("d12", 64, 1024): " (BASELINE configs[2])", ("d24", 32, 1024): " (BASELINE configs[3])",
-                                ("d48", 16, 1024): " (BASELINE configs[4])"}.get((args.model, B, T), ""),
-                   "global_batch": B, "seq_len": T, "tokens_per_step": B * T, "recompute": args.recompute,
-                   "gelu_fusion": args.gelu_fusion, "parallelism": "single GPU"},
+                                ("d48", 16, 1024): " (BASELINE configs[4])"}.get((model, B, T), ""),
+                   "global_batch": B, "seq_len": T, "tokens_per_step": B * T, "recompute": recompute,
+                   "gelu_fusion": gelu_fusion, "parallelism": "single GPU"},
         "mfu": float(mfu), "mfu_peak_tflops": PEAK_BF16_TFLOPS,
         "loss_first": float(losses[0]), "loss_last": float(losses[-1]),
         "roofline": roofline, "kernels_from_last_warmup_step": kernels,
     }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--seq", type=int, default=1024)
+    ap.add_argument("--model", default="d12")
+    ap.add_argument("--recompute", type=int, default=0)   # the reference's 124M recipe runs with -r 0 (scripts/run_gpt2_124M.sh)
+    ap.add_argument("--gelu-fusion", type=int, default=2)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-events", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the few steps of GPT-2 350M (B=32) and 1558M (B=16) that follow the headline measurement")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first launch one copy kernel of known size (128 MiB read, 256 MiB written): the yardstick for "
+                         "scaling FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this build runs the training step on ONE GPU only (no collectives are part of it); "
+              "use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    # the native driver and the reference's CPU trainer print their model headers with printf: send everything
+    # written to file descriptor 1 to stderr until the result line, so stdout carries exactly one JSON line
+    sys.stdout.flush()
+    real_stdout = os.dup(1)
+    os.dup2(2, 1)
+
+    import torch
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    pkg = package()
+    L = pkg.load("bf16")           # raises if the HIP library is not built: there is no other path
+    L.llmk_init(0)
+
+    if args.calibrate_copy:
+        n = 64 * 1024 * 1024
+        src = torch.zeros(n, dtype=torch.bfloat16, device="cuda")
+        dst = torch.empty(n, dtype=torch.float32, device="cuda")
+        L.llmk_copy_and_cast_to_f32(dst.data_ptr(), src.data_ptr(), n, 0, 0, 1, None)
+        torch.cuda.synchronize()
+        del src, dst
+
+    with SclkSampler() as step_clock:
+        out = run_workload(L, torch, args.model, args.batch, args.seq, args.recompute, args.gelu_fusion, args.steps,
+                           args.warmup, not args.no_kernel_events)
+    out = {"metric": METRIC, **out}
+
+    if not args.no_mfma_probe:
+        # the matrix cores by themselves, right after the timed region (same thermal state), with the driver's shader clock
+        # sampled meanwhile: what "peak" means on this machine at the clock it actually holds, next to the vendor figure
+        # every fraction above is priced against
+        ncu = C.c_int(0)
+        L.llmk_device_props(C.byref(ncu), None, None)
+        scratch = torch.zeros(16, dtype=torch.float32, device="cuda")
+        tf = C.c_double(0)
+        rates = []
+        with SclkSampler() as probe_clock:
+            for _ in range(30):
+                L.llmk_probe_mfma_peak(C.byref(tf), scratch.data_ptr(), None)
+                rates.append(tf.value)
+        del scratch
+        achieved = float(np.median(rates))
+        mhz = probe_clock.median()
+        out["mfma_probe"] = {
+            "compute_units": ncu.value, "achieved_tflops": achieved, "sclk_mhz": mhz,
+            "peak_at_clock_tflops": None if mhz is None else ncu.value * mhz * 1e6 * 4096 / 1e12,
+            "implied_clock_mhz": achieved * 1e12 / (ncu.value * 4096.0) / 1e6, "vendor_peak_tflops": PEAK_BF16_TFLOPS,
+            "note": "achieved: back-to-back v_mfma_f32_32x32x16_bf16 on register operands, 2 waves per SIMD, median of 30 "
+                    "runs of ~10 ms; sclk_mhz: median of the driver's current shader clock (pp_dpm_sclk) sampled every "
+                    "10 ms during those runs; peak_at_clock = compute_units x sclk x 4096 flop per CU and clock"}
+        out["sclk_mhz_during_timed_steps"] = step_clock.median()
+
+    if default_headline(args) and not args.no_other_configs:
+        # BASELINE configs[3] and configs[4], a few steps each, after and outside the headline measurement
+        out["other_configs"] = []
+        for model, b, lr in (("d24", 32, 3e-4), ("d48", 16, 6e-4)):          # learning rates of the reference's recipes
+            r = run_workload(L, torch, model, b, 1024, 1, 2, 3, 1, False, lr=lr)
+            out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
+                                                              "loss_first", "loss_last")})
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     C.CDLL(None).fflush(None)
@@ -236,10 +353,6 @@ def main():
     os.dup2(real_stdout, 1)
     os.close(real_stdout)
     print(json.dumps(out), flush=True)
-
-
-def ctypes_float(x):
-    return C.c_float(x)
 
 
 if __name__ == "__main__":

@@ -68,6 +68,12 @@ void llmk_profile_get(int i, char* name64, int* calls, double* ms, double* flops
  * bandwidth. Any alignment and size. */
 void llmk_zero(void* ptr, size_t bytes, void* stream);
 
+/* Measurement aid, no counterpart in the reference (its mfu.h tabulates vendor peaks, llmc/mfu.h:43-147): the
+ * TFLOP/s the matrix cores of this GPU deliver to back-to-back bf16 MFMAs on register operands (non-trivial values), two
+ * waves per SIMD, for about ten milliseconds - i.e. CUs x 4096 flop per CU and clock x the clock the chip holds under that
+ * load. scratch: one float of device memory. Synchronises the stream. The fp32 library returns zero. */
+void llmk_probe_mfma_peak(double* tflops, float* scratch, void* stream);
+
 /* ---- encoder (llmc/encoder.cuh) ---------------------------------------------------------- */
 
 /* encoder_forward, llmc/encoder.cuh:157. out[b,t,:] = wte[inp[b,t],:] + wpe[t,:] */

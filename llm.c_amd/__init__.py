@@ -43,6 +43,7 @@ KERNEL_ABI = {
     "llmk_profile_enable": (None, [i32]),
     "llmk_profile_only": (None, [C.c_char_p]),
     "llmk_zero": (None, [vp, C.c_size_t, vp]),
+    "llmk_probe_mfma_peak": (None, [C.POINTER(C.c_double), vp, vp]),
     "llmk_profile_reset": (None, []),
     "llmk_profile_count": (i32, []),
     "llmk_profile_get": (None, [i32, C.c_char_p, ip, C.POINTER(C.c_double), C.POINTER(C.c_double), C.POINTER(C.c_double)]),

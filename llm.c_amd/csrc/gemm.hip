@@ -555,9 +555,68 @@ int bias_grad_ny(int OC) {
 
 bool aligned16(const void* p) { return ((uintptr_t)p % 16) == 0; }
 
+#if !defined(LLMK_FP32)
+// What the matrix cores deliver when nothing else is in the way: every wave issues independent chains of
+// v_mfma_f32_32x32x16_bf16 on operands it holds in registers (non-trivial values: the clock the chip sustains depends on
+// the data), two waves per SIMD.
+__global__ void __launch_bounds__(512)
+mfma_peak_kernel(float* __restrict__ sink, int iters) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const int lane = threadIdx.x & 63;
+    bf16x8 a, b;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        a[e] = (__bf16)(0.03125f * (float)(((lane * 8 + e) * 37 + blockIdx.x) % 61 - 30));
+        b[e] = (__bf16)(0.0625f * (float)(((lane * 8 + e) * 53 + threadIdx.x) % 59 - 29));
+    }
+    f32x16 acc[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[c][r] = 0.f;
+    for (int it = 0; it < iters; it++) {
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int c = 0; c < 4; c++) acc[c] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, acc[c], 0, 0, 0);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int c = 0; c < 4; c++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) s += acc[c][r];
+    if (s == 12345.678f) sink[0] = s;                                   // keeps the chains alive
+#endif
+}
+#endif
+
 }  // namespace
 
 extern "C" {
+
+void llmk_probe_mfma_peak(double* tflops, float* scratch, void* stream) {
+    if (tflops) *tflops = 0.0;
+#if !defined(LLMK_FP32)
+    if (llmk::failed()) return;
+    LLMK_REQUIRE(scratch != nullptr, "probe_mfma_peak: one float of device scratch is required");
+    hipStream_t st = (hipStream_t)stream;
+    const int num_cu = llmk::device_info().num_cu, iters = 16384;       // 16 MFMAs per iteration and wave
+    hipEvent_t e0, e1;
+    HIP_CHECK(hipEventCreate(&e0));
+    HIP_CHECK(hipEventCreate(&e1));
+    mfma_peak_kernel<<<num_cu, 512, 0, st>>>(scratch, 1024);            // warm-up: the clock settles under matrix load
+    HIP_CHECK(hipEventRecord(e0, st));
+    mfma_peak_kernel<<<num_cu, 512, 0, st>>>(scratch, iters);
+    HIP_CHECK(hipEventRecord(e1, st));
+    HIP_CHECK(hipEventSynchronize(e1));
+    float ms = 0.f;
+    HIP_CHECK(hipEventElapsedTime(&ms, e0, e1));
+    HIP_CHECK(hipEventDestroy(e0));
+    HIP_CHECK(hipEventDestroy(e1));
+    const double flops = (double)num_cu * 8.0 * iters * 16.0 * 32768.0;    // 8 waves per workgroup, 2*32*32*16 flop per MFMA
+    if (ms > 0.f && tflops) *tflops = flops / (ms * 1e-3) / 1e12;
+#endif
+}
 
 void llmk_matmul_forward(void* out, const void* inp, const void* weight, const void* bias, int B, int T, int C,
                          int OC, void* stream, void* pre_gelu, int gelu_fusion) {
