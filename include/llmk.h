@@ -155,6 +155,19 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                              int B, int T, int NH, int C, void* stream);
 
+/* attention_forward, llmc/attention.cuh:195: the launcher of reference builds without cuDNN, same argument order.
+ * inp (B,T,3C) Q, K, V as the qkv projection wrote them; out (B,T,C). qkvr (B*T*3C elements) and att (B*NH*T*T elements)
+ * are the buffers the reference keeps for its backward pass; this library keeps other things in them (qkvr: a copy of inp
+ * as it came; att: the fp32 log-sum-exp of every row in its first B*NH*T*4 bytes, which needs T*sizeof(floatX) >= 4), so
+ * they are only meaningful to llmk_attention_backward_fallback. inp is left intact (the reference overwrites it). */
+void llmk_attention_forward_fallback(void* out, void* qkvr, void* att, void* inp, int B, int T, int C, int NH, void* stream);
+
+/* attention_backward, llmc/attention.cuh:239, same argument order. dinp (B,T,3C) is overwritten with the gradient of
+ * the un-permuted Q, K, V; qkvr and att as llmk_attention_forward_fallback left them; scratch (B*T*C elements) receives
+ * the forward output again (the reference's signature does not pass it); dqkvr and datt are not touched. */
+void llmk_attention_backward_fallback(void* dinp, void* dqkvr, void* datt, void* scratch, const void* dout, const void* qkvr,
+                                      const void* att, int B, int T, int C, int NH, void* stream);
+
 /* The same operation for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc). It has no counterpart in the reference. The rowsum(dO*O) vector lives in a
  * 4 MiB array that is part of the library's code object on every GPU instead of the grow-only workspace, so the call
@@ -201,6 +214,17 @@ void llmk_adamw_update(void* params_memory, float* master_params_memory, const v
                        float* v_memory, size_t num_parameters, ptrdiff_t w_stride, ptrdiff_t g_stride,
                        ptrdiff_t s_stride, int num_slices, float learning_rate, float beta1, float beta2, int t,
                        float eps, float weight_decay, float grad_scale, unsigned int seed, void* stream);
+/* Several tensors in one launch; no counterpart in the reference, whose gpt2_update launches adamw_update once per
+ * tensor (train_gpt2.cu:1056-1106; ten of GPT-2's sixteen tensors are a few KB). All five arenas share one layout: tensor
+ * i starts offsets[i] elements into each of them and has num_slices[i] contiguous slices of sizes[i] elements, its own
+ * weight decay and seed. Same arithmetic and the same stochastic-rounding words as count calls of llmk_adamw_update with
+ * strides equal to sizes[i]. Returns 1 when it ran; 0 (nothing done) when the tensors do not suit it - more than 16,
+ * sizes or offsets not multiples of 16 bytes of floatX, misaligned arenas - and the caller falls back to per-tensor calls. */
+int llmk_adamw_update_multi(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                            const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                            const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
+                            void* stream);
+
 /* init_from_master, llmc/adamw.cuh:90. params = stochastic_round(master), same noise as above. */
 void llmk_init_from_master(void* params_memory, const float* master_params_memory, size_t num_parameters,
                            ptrdiff_t w_stride, ptrdiff_t s_stride, int num_slices, unsigned int seed,

@@ -60,6 +60,8 @@ KERNEL_ABI = {
     "llmk_gelu_backward_bias": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),
     "llmk_attention_forward": (None, [vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_attention_backward": (None, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "llmk_attention_forward_fallback": (None, [vp, vp, vp, vp, i32, i32, i32, i32, vp]),
+    "llmk_attention_backward_fallback": (None, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_attention_backward_static": (None, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_gelu_forward": (None, [vp, vp, i32, vp]),
     "llmk_gelu_backward_inplace": (None, [vp, vp, i32, vp]),
@@ -68,6 +70,8 @@ KERNEL_ABI = {
     "llmk_global_norm_squared": (None, [vp, vp, sz, pd, i32, i32, i32, vp]),
     "llmk_global_sum_deterministic": (None, [vp, vp, i32, vp]),
     "llmk_adamw_update": (None, [vp, vp, vp, vp, vp, sz, pd, pd, pd, i32, f32, f32, f32, i32, f32, f32, f32, u32, vp]),
+    "llmk_adamw_update_multi": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, i32,
+                                      C.c_float, C.c_float, vp]),
     "llmk_init_from_master": (None, [vp, vp, sz, pd, pd, i32, u32, vp]),
     "llmk_copy_and_cast_to_f32": (None, [vp, vp, sz, pd, pd, i32, vp]),
 }

@@ -1277,6 +1277,28 @@ void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, co
     attention_backward_impl(dqkvr, dout, qkvr, o, stats, B, T, NH, C, stream, nullptr);
 }
 
+// The reference's launchers for builds without cuDNN (llmc/attention.cuh:195, :239) keep a permuted copy of Q, K, V and
+// the (B,NH,T,T) probabilities between the passes. Here the same buffers carry what the flash kernels need instead: qkvr
+// holds Q, K, V as they came (B,T,3,NH,hs), and the first B*NH*T*4 bytes of att hold the fp32 log-sum-exp of every row.
+void llmk_attention_forward_fallback(void* out, void* qkvr, void* att, void* inp, int B, int T, int C, int NH, void* stream) {
+    if (llmk::failed()) return;
+    if ((size_t)B * T == 0) return;
+    LLMK_REQUIRE((size_t)T * sizeof(floatX) >= sizeof(float), "attention_forward: T=%d too short for the statistics to fit the att buffer", T);
+    LLMK_REQUIRE(((uintptr_t)att % 4) == 0, "attention_forward: att must be 4-byte aligned");
+    HIP_CHECK(hipMemcpyAsync(qkvr, inp, (size_t)B * T * 3 * C * sizeof(floatX), hipMemcpyDeviceToDevice, (hipStream_t)stream));
+    llmk_attention_forward(out, (float*)att, qkvr, B, T, NH, C, stream);
+}
+
+void llmk_attention_backward_fallback(void* dinp, void* dqkvr, void* datt, void* scratch, const void* dout, const void* qkvr,
+                                      const void* att, int B, int T, int C, int NH, void* stream) {
+    if (llmk::failed()) return;
+    (void)dqkvr; (void)datt;                                     // the flash kernels need neither
+    if ((size_t)B * T == 0) return;
+    // the output of the forward pass is not among the arguments: it is formed again, in scratch (B*T*C elements)
+    llmk_attention_forward(scratch, nullptr, qkvr, B, T, NH, C, stream);
+    llmk_attention_backward(dinp, dout, qkvr, scratch, (const float*)att, B, T, NH, C, stream);
+}
+
 void llmk_attention_backward_static(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                                     int B, int T, int NH, int C, void* stream) {
     if (llmk::failed()) return;

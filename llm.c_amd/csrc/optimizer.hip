@@ -74,6 +74,65 @@ adamw_vec_kernel(floatX* __restrict__ params, float* __restrict__ master, const 
     }
 }
 
+// All tensors of a model in one launch: block b belongs to the tensor whose range of blocks contains it, then to a slice
+// and a 2048-element piece of that slice. Same arithmetic, same noise words as one adamw_vec_kernel launch per tensor.
+struct AdamTensorTable {
+    static constexpr int MAX = 16;
+    int count;
+    unsigned first_block[MAX + 1];        // first_block[count] = grid size
+    unsigned blocks_per_slice[MAX];
+    unsigned long long offset[MAX];       // elements from the start of every arena
+    unsigned long long n[MAX];            // elements per slice (slices are contiguous: stride n)
+    float wd[MAX];
+    unsigned seed[MAX];
+};
+__global__ void __launch_bounds__(256)
+adamw_multi_kernel(floatX* __restrict__ params, float* __restrict__ master, const floatX* __restrict__ grads,
+                   float* __restrict__ m, float* __restrict__ v, AdamTensorTable tab, AdamArgs a) {
+    int ti = 0;
+    while (ti + 1 < tab.count && blockIdx.x >= tab.first_block[ti + 1]) ti++;      // wave-uniform, at most 15 steps
+    const unsigned local = blockIdx.x - tab.first_block[ti];
+    const int slice = (int)(local / tab.blocks_per_slice[ti]);
+    const size_t n = tab.n[ti];
+    const size_t i = ((size_t)(local % tab.blocks_per_slice[ti]) * 256 + threadIdx.x) * VN;
+    if (i >= n) return;
+    const size_t base = tab.offset[ti] + (size_t)slice * n + i;
+    a.wd = tab.wd[ti];
+    a.seed = tab.seed[ti];
+    vecX g = ld_vec_nt(grads + base);
+    vecX p;
+    if (!master) p = ld_vec(params + base);
+    float mm[VN], vv[VN], ms[VN];
+#pragma unroll
+    for (int q = 0; q < VN / 4; q++) {
+        vecF t = ld_vec(m + base + q * 4), u = ld_vec(v + base + q * 4);
+#pragma unroll
+        for (int k = 0; k < 4; k++) { mm[q * 4 + k] = t[k]; vv[q * 4 + k] = u[k]; }
+        if (master) {
+            vecF w = ld_vec(master + base + q * 4);
+#pragma unroll
+            for (int k = 0; k < 4; k++) ms[q * 4 + k] = w[k];
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < VN; k++) {
+        float old = master ? ms[k] : to_f32(p[k]);
+        float np = adam_one(to_f32(g[k]), mm[k], vv[k], old, a);
+        ms[k] = np;
+        stochastic_store(np, &p[k], adamw_noise(i + k, slice, a.seed));
+    }
+    st_vec(params + base, p);
+#pragma unroll
+    for (int q = 0; q < VN / 4; q++) {
+        vecF t, u, w;
+#pragma unroll
+        for (int k = 0; k < 4; k++) { t[k] = mm[q * 4 + k]; u[k] = vv[q * 4 + k]; w[k] = ms[q * 4 + k]; }
+        st_vec(m + base + q * 4, t);
+        st_vec(v + base + q * 4, u);
+        if (master) st_vec(master + base + q * 4, w);
+    }
+}
+
 __global__ void __launch_bounds__(256)
 adamw_scalar_kernel(floatX* __restrict__ params, float* __restrict__ master, const floatX* __restrict__ grads,
                     float* __restrict__ m, float* __restrict__ v, size_t n, ptrdiff_t w_stride, ptrdiff_t g_stride,
@@ -176,6 +235,36 @@ void llmk_adamw_update(void* params_memory, float* master, const void* grads_mem
                                                   w_stride, g_stride, s_stride, a);
     }
     LAUNCH_CHECK();
+}
+
+int llmk_adamw_update_multi(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                            const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                            const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
+                            void* stream) {
+    if (llmk::failed()) return 0;
+    if (count <= 0 || count > AdamTensorTable::MAX) return 0;
+    auto al = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
+    if (!(al(params_memory) && al(grads_memory) && al(m) && al(v) && (!master || al(master)))) return 0;
+    AdamTensorTable tab{};
+    tab.count = count;
+    unsigned long long blocks = 0;
+    double elems = 0;
+    for (int i = 0; i < count; i++) {
+        if (sizes[i] == 0 || num_slices[i] <= 0 || sizes[i] % VN != 0 || offsets[i] % VN != 0) return 0;
+        tab.first_block[i] = (unsigned)blocks;
+        tab.blocks_per_slice[i] = (unsigned)CEIL_DIV(sizes[i] / VN, (size_t)256);
+        tab.offset[i] = offsets[i]; tab.n[i] = sizes[i]; tab.wd[i] = weight_decays[i]; tab.seed[i] = seeds[i];
+        blocks += (unsigned long long)tab.blocks_per_slice[i] * num_slices[i];
+        elems += (double)sizes[i] * num_slices[i];
+        if (blocks > 0x7fffffffull) return 0;
+    }
+    tab.first_block[count] = (unsigned)blocks;
+    AdamArgs a{lr, beta1, beta2, 1.0f - powf(beta1, (float)t), 1.0f - powf(beta2, (float)t), eps, 0.f, grad_scale, 0u};
+    hipStream_t st = (hipStream_t)stream;
+    llmk::ProfScope prof("adamw_update", 0, elems * (master ? 2.0 * sizeof(floatX) + 24.0 : 3.0 * sizeof(floatX) + 16.0), st);
+    adamw_multi_kernel<<<(unsigned)blocks, 256, 0, st>>>((floatX*)params_memory, master, (const floatX*)grads_memory, m, v, tab, a);
+    LAUNCH_CHECK();
+    return 1;
 }
 
 void llmk_init_from_master(void* params_memory, const float* master, size_t n, ptrdiff_t w_stride,

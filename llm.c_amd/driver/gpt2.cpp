@@ -613,6 +613,29 @@ void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, fl
         hipCheck(hipMemsetAsync(m->v_memory, 0, m->num_parameters * sizeof(float), st));
     }
     m->rng_state_last_update = m->rng_state;
+    // every tensor in one launch where the library takes them so (same results as the per-tensor calls below, which the
+    // reference makes: ten of the sixteen tensors are a few KB and cost a launch each); the seeds are drawn in the same order
+    if (!init_from_master_only && !(init_state && m->master_weights != nullptr)) {
+        size_t offsets[NUM_PARAMETER_TENSORS], sizes[NUM_PARAMETER_TENSORS];
+        int slices[NUM_PARAMETER_TENSORS];
+        float wds[NUM_PARAMETER_TENSORS];
+        unsigned int seeds[NUM_PARAMETER_TENSORS];
+        unsigned long long rng = m->rng_state;
+        for (int i = 0; i < NUM_PARAMETER_TENSORS; i++) {
+            seeds[i] = llmk::random_u32(&rng);
+            ShardInfo tensor = tensor_at_layer(m, 0, i);
+            offsets[i] = tensor.offset; sizes[i] = tensor.size;
+            slices[i] = (i < 2 || i > 13) ? 1 : m->config.num_layers;
+            wds[i] = (i == 0 || i == 1 || i == 4 || i == 6 || i == 10 || i == 12) ? weight_decay : 0.0f;
+        }
+        if (llmk_adamw_update_multi(m->params_memory, m->master_weights, m->grads_memory, m->m_memory, m->v_memory,
+                                    NUM_PARAMETER_TENSORS, offsets, sizes, slices, wds, seeds, learning_rate, beta1, beta2, t,
+                                    eps, grad_scale, st)) {
+            m->rng_state = rng;
+            hipCheck(hipStreamSynchronize(st));
+            return;
+        }
+    }
     for (int i = 0; i < NUM_PARAMETER_TENSORS; i++) {
         unsigned int seed = llmk::random_u32(&m->rng_state);
         int num_layers = (i < 2 || i > 13) ? 1 : m->config.num_layers;

@@ -424,6 +424,39 @@ def test_attention_forward_backward(precision, B, T, NH):
 
 
 @pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("B,T,NH", [(2, 128, 3), (1, 200, 2)])
+def test_attention_fallback_launchers(precision, B, T, NH):
+    """The launcher pair of reference builds without cuDNN (llmc/attention.cuh:195, :239), in its argument order: same
+    bits as the flash pair, from the buffers that signature provides (qkvr, att, scratch), against the oracle."""
+    import torch
+    L = G.lib(precision)
+    dt = G.torch_dtype(precision)
+    qkv, g, ro, rlse, rd, Cc = attention_case(precision, B, T, NH, seed=7)
+    d_inp, d_g = G.dev(qkv, precision), G.dev(g, precision)
+    d_o, d_stats = torch.zeros((B, T, Cc), dtype=dt, device="cuda"), torch.zeros((B, NH, T), dtype=torch.float32, device="cuda")
+    L.llmk_attention_forward(G.ptr(d_o), G.ptr(d_stats), G.ptr(d_inp), B, T, NH, Cc, None)
+    d_want = torch.zeros((B, T, 3 * Cc), dtype=dt, device="cuda")
+    L.llmk_attention_backward(G.ptr(d_want), G.ptr(d_g), G.ptr(d_inp), G.ptr(d_o), G.ptr(d_stats), B, T, NH, Cc, None)
+    d_qkvr = torch.zeros((B, T, 3 * Cc), dtype=dt, device="cuda")
+    d_att = torch.full((B, NH, T, T), 9.0, dtype=dt, device="cuda")
+    d_o2 = torch.zeros((B, T, Cc), dtype=dt, device="cuda")
+    inp_copy = d_inp.clone()
+    L.llmk_attention_forward_fallback(G.ptr(d_o2), G.ptr(d_qkvr), G.ptr(d_att), G.ptr(inp_copy), B, T, Cc, NH, None)
+    inp_copy.fill_(5.0)                                     # the reference's driver reuses this buffer right away
+    d_dinp = torch.full((B, T, 3 * Cc), 3.0, dtype=dt, device="cuda")
+    d_dqkvr, d_datt = torch.zeros_like(d_qkvr), torch.zeros_like(d_att)
+    d_scratch = torch.full((B, T, Cc), 7.0, dtype=dt, device="cuda")
+    L.llmk_attention_backward_fallback(G.ptr(d_dinp), G.ptr(d_dqkvr), G.ptr(d_datt), G.ptr(d_scratch), G.ptr(d_g), G.ptr(d_qkvr),
+                                       G.ptr(d_att), B, T, Cc, NH, None)
+    G.sync()
+    assert torch.equal(d_o2, d_o) and torch.equal(d_dinp, d_want)
+    close(G.host(d_o2), ro, **tol(precision, 1e-5, bf16_atol=2e-2), what="out")
+    scale = np.abs(rd).max()
+    close(G.host(d_dinp), rd, **tol(precision, 1e-4 * scale, bf16_rel=1.0 / 32, bf16_atol=2e-2 * scale), what="dinp")
+    G.check_no_error(L)
+
+
+@pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("hs", [32, 80, 96, 128])
 @pytest.mark.parametrize("B,T,NH", [(2, 96, 2), (1, 130, 3)])
 def test_attention_other_head_sizes(precision, hs, B, T, NH):
@@ -444,6 +477,58 @@ def test_attention_other_head_sizes(precision, hs, B, T, NH):
 
 
 # ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("use_master", [True, False])
+def test_adamw_update_multi_is_the_per_tensor_update(precision, use_master):
+    """Sixteen tensors in one launch against sixteen launches: the same bits in every arena, including the noise words
+    of the stochastic rounding (per slice, per element index inside the slice)."""
+    import torch
+    L = G.lib(precision)
+    rs = np.random.RandomState(5)
+    sizes = [int(x) * 8 for x in rs.randint(1, 700, 16)]
+    sizes[0], sizes[5] = 300000, 8                         # one large tensor, one of a single vector
+    slices = [1, 1] + [int(x) for x in rs.randint(1, 5, 12)] + [1, 1]
+    wds = [0.1 if i in (0, 1, 4, 6, 10, 12) else 0.0 for i in range(16)]
+    seeds = [int(x) for x in rs.randint(0, 2 ** 31, 16)]
+    offsets = np.cumsum([0] + [sz * sl for sz, sl in zip(sizes, slices)])
+    tot = int(offsets[-1])
+    p0 = G.rounded(rnd(tot, 0, 0.05), precision); g = G.rounded(rnd(tot, 1, 0.01), precision)
+    m0, v0 = rnd(tot, 2, 0.01), np.abs(rnd(tot, 3, 1e-4))
+    master0 = (p0 + rnd(tot, 4, 1e-4)).astype(np.float32) if use_master else None
+    hp = (1e-3, 0.9, 0.95, 3, 1e-8)
+    gs = 0.5
+    X = 2 if precision == "bf16" else 4
+
+    def arenas():
+        return [G.dev(p0, precision), (G.dev(master0) if use_master else None), G.dev(g, precision), G.dev(m0), G.dev(v0)]
+
+    a = arenas()
+    for i in range(16):
+        o = int(offsets[i])
+        ptrs = [None if t is None else CT.c_void_p(t.data_ptr() + o * (X if k in (0, 2) else 4)) for k, t in enumerate(a)]
+        L.llmk_adamw_update(ptrs[0], ptrs[1], ptrs[2], ptrs[3], ptrs[4], sizes[i], sizes[i], sizes[i], sizes[i], slices[i],
+                            hp[0], hp[1], hp[2], hp[3], hp[4], wds[i], gs, seeds[i], None)
+    b = arenas()
+    off_a, size_a = np.array(offsets[:16], np.uint64), np.array(sizes, np.uint64)
+    sl_a, wd_a, seed_a = np.array(slices, np.int32), np.array(wds, np.float32), np.array(seeds, np.uint32)
+    vp = lambda x: x.ctypes.data_as(CT.c_void_p)
+    ran = L.llmk_adamw_update_multi(G.ptr(b[0]), G.ptr(b[1]), G.ptr(b[2]), G.ptr(b[3]), G.ptr(b[4]), 16, vp(off_a), vp(size_a),
+                                    vp(sl_a), vp(wd_a), vp(seed_a), hp[0], hp[1], hp[2], hp[3], hp[4], gs, None)
+    assert ran == 1
+    G.sync()
+    for x, y in zip(a, b):
+        if x is not None:
+            assert torch.equal(x, y)
+    assert not torch.equal(a[0], G.dev(p0, precision))     # and something happened
+    # tensors the single launch cannot take are refused, not mangled
+    size_a[3] += 1
+    assert L.llmk_adamw_update_multi(G.ptr(b[0]), G.ptr(b[1]), G.ptr(b[2]), G.ptr(b[3]), G.ptr(b[4]), 16, vp(off_a), vp(size_a),
+                                     vp(sl_a), vp(wd_a), vp(seed_a), hp[0], hp[1], hp[2], hp[3], hp[4], gs, None) == 0
+    G.sync()
+    assert torch.equal(a[0], b[0])
+    G.check_no_error(L)
+
+
 @pytest.mark.parametrize("precision", PRECS)
 @pytest.mark.parametrize("use_master", [True, False])
 def test_adamw_update(precision, use_master):
