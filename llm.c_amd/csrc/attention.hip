@@ -365,14 +365,18 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
 // inline asm the reads of the tile in use do not wait for the tile in flight. Same arithmetic in the same order as
 // fa_forward_kernel: the two give identical bits.
 __global__ void __launch_bounds__(256, 4)
-fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH) {
+fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const floatX* __restrict__ qkv, int T, int NH, int nq) {
     constexpr int NWAVES = 4;
     __shared__ __attribute__((aligned(1024))) char sK[2][SW_TILE];
     __shared__ __attribute__((aligned(1024))) char sV[2][SW_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
     int tile_x, bh;
     fa_block_coords(tile_x, bh);
-    const int qt = gridDim.x - 1 - tile_x;              // longest rows first
+    // A workgroup takes TWO tiles of 128 queries of its head, nq - 1 - x and then x (one when they coincide): together
+    // they walk nq + 1 pairs of key tiles whatever x is, so every workgroup of the launch does the same work, and the
+    // second tile's first keys are already on their way when the first tile is stored.
+    const int qt_first = nq - 1 - tile_x, qt_second = tile_x;
+    const int nphase = qt_first == qt_second ? 1 : 2;
     const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
@@ -385,111 +389,121 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
     const floatX* vbase = fa_uniform(base + 2 * C);
     fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
     fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
-    constexpr int GQ = 32 * NWAVES;                       // queries per workgroup
-    const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
+    constexpr int GQ = 32 * NWAVES;                       // queries per tile
     const float c = 0.125f * LOG2E;                       // 1/sqrt(64) folded into the exp2 argument
-
-    bf16x8 qf[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-        if (my_q < T) qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
-        else
-#pragma unroll
-            for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
-    }
-    f32x16 o[2];
-#pragma unroll
-    for (int d = 0; d < 2; d++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) o[d][r] = 0.f;
-    float m = -INFINITY;
     const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    // The softmax denominator is accumulated by the matrix cores, which have cycles to spare here: a ones operand
-    // in place of V makes every row of this accumulator the sum over keys of the (bf16-rounded) probabilities of
-    // the lane's query - the same rounded values that multiply V.
-    f32x16 lacc = zero;
     bf16x8 ones;
 #pragma unroll
     for (int e = 0; e < 8; e++) ones[e] = (__bf16)1.0f;
+    int buf = 0;                                          // the buffer that holds the key tile of the coming step
 
-    const int last_q = min(qt * GQ + GQ - 1, T - 1);
-    const int n_kt = last_q / 64 + 1;
-    fa_tiles_landed();
-    __syncthreads();
-
-    for (int j = 0; j < n_kt; j++) {
-        const unsigned tk = fa_lds_addr(sK[j & 1]), tv = fa_lds_addr(sV[j & 1]);
-        if (j + 1 < n_kt) {                              // the other buffer was last read before the barrier that ended step j - 1
-            fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[(j + 1) & 1]), uwave);
-            fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[(j + 1) & 1]), uwave);
-        }
-        auto kfrag = [&](int row0, int s) -> bf16x8 { return fa_frag_rows(tk, la, row0, s); };
-        auto vfrag = [&](int kb, int col0) -> bf16x8 { return fa_frag_cols(tv, la, kb, col0); };
-        if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
-            // S^T for both 32-key blocks, the two accumulation chains interleaved
-            f32x16 sacc[2];
-            sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, 0), qf[0], zero, 0, 0, 0);
-            sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, 0), qf[0], zero, 0, 0, 0);
+    for (int phase = 0; phase < nphase; phase++) {
+        const int qt = phase == 0 ? qt_first : qt_second;
+        const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
+        bf16x8 qf[4];
 #pragma unroll
-            for (int s = 1; s < 4; s++) {
-                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, s), qf[s], sacc[0], 0, 0, 0);
-                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, s), qf[s], sacc[1], 0, 0, 0);
+        for (int s = 0; s < 4; s++) {
+            if (my_q < T) qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+            else
+#pragma unroll
+                for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
+        }
+        f32x16 o[2];
+#pragma unroll
+        for (int d = 0; d < 2; d++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) o[d][r] = 0.f;
+        float m = -INFINITY;
+        // The softmax denominator is accumulated by the matrix cores, which have cycles to spare here: a ones operand
+        // in place of V makes every row of this accumulator the sum over keys of the (bf16-rounded) probabilities of
+        // the lane's query - the same rounded values that multiply V.
+        f32x16 lacc = zero;
+
+        const int last_q = min(qt * GQ + GQ - 1, T - 1);
+        const int n_kt = last_q / 64 + 1;
+        // the wave's own rows have arrived (and, for the first tile, the first keys; the second tile's first keys were
+        // awaited by the step that ended the first tile): after this the only loads in flight are tile requests
+        fa_tiles_landed();
+        if (phase == 0) __syncthreads();
+
+        for (int j = 0; j < n_kt; j++) {
+            const unsigned tk = fa_lds_addr(sK[buf]), tv = fa_lds_addr(sV[buf]);
+            buf ^= 1;
+            if (j + 1 < n_kt) {                          // the other buffer was last read before the barrier that ended the previous step
+                fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[buf]), uwave);
+                fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[buf]), uwave);
+            } else if (phase + 1 < nphase) {             // the second tile starts over at the head's first keys
+                fa_tile_request(la, kbase, fa_lds_addr(sK[buf]), uwave);
+                fa_tile_request(la, vbase, fa_lds_addr(sV[buf]), uwave);
             }
-            if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
-                asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
+            auto kfrag = [&](int row0, int s) -> bf16x8 { return fa_frag_rows(tk, la, row0, s); };
+            auto vfrag = [&](int kb, int col0) -> bf16x8 { return fa_frag_cols(tv, la, kb, col0); };
+            if (64 * j <= qw0 + 31) {                          // else: every key of this tile is in the future of this wave
+                // S^T for both 32-key blocks, the two accumulation chains interleaved
+                f32x16 sacc[2];
+                sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, 0), qf[0], zero, 0, 0, 0);
+                sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, 0), qf[0], zero, 0, 0, 0);
+#pragma unroll
+                for (int s = 1; s < 4; s++) {
+                    sacc[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(0, s), qf[s], sacc[0], 0, 0, 0);
+                    sacc[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kfrag(32, s), qf[s], sacc[1], 0, 0, 0);
+                }
+                if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
+                    asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
+#pragma unroll
+                    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++)
+                            if (64 * j + 32 * kb + acc_row(r, lane) > my_q) sacc[kb][r] = -INFINITY;
+                }
+                float mx = fmaxf(sacc[0][0], sacc[1][0]);
+#pragma unroll
+                for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
+                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                const float m_top = fmaxf(m, mx * c);
+                const bool outgrown = m_top > m + FA_MAX_SLACK;
+                if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
+                    asm volatile("" ::: "memory");
+                    // every row decides for itself, so that what a row computes depends on that row's scores alone
+                    const float m_new = outgrown ? m_top : m;
+                    const float alpha = fast_exp2(m - m_new);
+                    m = m_new;
+#pragma unroll
+                    for (int r = 0; r < 16; r++) lacc[r] *= alpha;
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+#pragma unroll
+                        for (int r = 0; r < 16; r++) o[d][r] *= alpha;
+                }
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        if (64 * j + 32 * kb + acc_row(r, lane) > my_q) sacc[kb][r] = -INFINITY;
+                        sacc[kb][r] = fast_exp2(fmaf(sacc[kb][r], c, -m));
+#pragma unroll
+                for (int s2 = 0; s2 < 4; s2++) {
+                    const bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
+                    lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, lacc, 0, 0, 0);       // every row: sum over keys of P
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+                        o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(16 * s2, 32 * d), pf, o[d], 0, 0, 0);
+                }
             }
-            float mx = fmaxf(sacc[0][0], sacc[1][0]);
-#pragma unroll
-            for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
-            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-            const float m_top = fmaxf(m, mx * c);
-            const bool outgrown = m_top > m + FA_MAX_SLACK;
-            if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
-                asm volatile("" ::: "memory");
-                // every row decides for itself, so that what a row computes depends on that row's scores alone
-                const float m_new = outgrown ? m_top : m;
-                const float alpha = fast_exp2(m - m_new);
-                m = m_new;
-#pragma unroll
-                for (int r = 0; r < 16; r++) lacc[r] *= alpha;
-#pragma unroll
-                for (int d = 0; d < 2; d++)
-#pragma unroll
-                    for (int r = 0; r < 16; r++) o[d][r] *= alpha;
-            }
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    sacc[kb][r] = fast_exp2(fmaf(sacc[kb][r], c, -m));
-#pragma unroll
-            for (int s2 = 0; s2 < 4; s2++) {
-                const bf16x8 pf = pack_acc(sacc[s2 >> 1], s2 & 1);
-                lacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ones, pf, lacc, 0, 0, 0);       // every row: sum over keys of P
-#pragma unroll
-                for (int d = 0; d < 2; d++)
-                    o[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vfrag(16 * s2, 32 * d), pf, o[d], 0, 0, 0);
-            }
+            fa_tiles_landed();
+            __syncthreads();
         }
-        fa_tiles_landed();
-        __syncthreads();
-    }
 
-    const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
-    if (my_q < T) {
-        const float inv = 1.0f / l;
-        floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
+        const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
+        if (my_q < T) {
+            const float inv = 1.0f / l;
+            floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
 #pragma unroll
-        for (int d = 0; d < 2; d++)
+            for (int d = 0; d < 2; d++)
 #pragma unroll
-            for (int g = 0; g < 4; g++)
-                store4(dst + 32 * d + 8 * g + 4 * half, o[d][4 * g] * inv, o[d][4 * g + 1] * inv, o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
-        if (stats && half == 0) stats[((size_t)b * NH + h) * T + my_q] = (m + __log2f(l)) * 0.6931471805599453f;
+                for (int g = 0; g < 4; g++)
+                    store4(dst + 32 * d + 8 * g + 4 * half, o[d][4 * g] * inv, o[d][4 * g + 1] * inv, o[d][4 * g + 2] * inv, o[d][4 * g + 3] * inv);
+            if (stats && half == 0) stats[((size_t)b * NH + h) * T + my_q] = (m + __log2f(l)) * 0.6931471805599453f;
+        }
     }
 }
 
@@ -656,15 +670,20 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
 // Same computation with the Q / dO tiles brought in by direct-to-LDS loads (needs T % 64 == 0): no staging registers.
 __global__ void __launch_bounds__(256)
 fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
-                        const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH) {
+                        const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH, int nk) {
     __shared__ __attribute__((aligned(1024))) char sQ[2][SW_TILE];
     __shared__ __attribute__((aligned(1024))) char sdO[2][SW_TILE];
     extern __shared__ __attribute__((aligned(16))) float sStat[];   // [2][T]: log-sum-exp (in log2 units) and rowsum(dO*O) of every query of this head
     float* sLall = sStat;
     float* sDall = sStat + T;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
-    int kt, bh;
-    fa_block_coords(kt, bh);
+    int tile_x, bh;
+    fa_block_coords(tile_x, bh);
+    // Two tiles of 128 keys per workgroup, x (the one with more queries after it) and then nk - 1 - x (one when they
+    // coincide): equal work for every workgroup of the launch, and the second tile's first queries are on their way
+    // when the first tile is stored.
+    const int kt_first = tile_x, kt_second = nk - 1 - tile_x;
+    const int nphase = kt_first == kt_second ? 1 : 2;
     const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
@@ -672,109 +691,120 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
     const floatX* dobase = dout + (size_t)b * T * C + h * HS;
     const float* lbase = stats + ((size_t)b * NH + h) * T;
     const float* dbase = Dsum + ((size_t)b * NH + h) * T;
-    const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
     const float c = 0.125f * LOG2E;
     // the first Q and dO tiles are requested before anything else: they travel while the wave fetches its own rows
-    const int q_first = (kt * 128) / 64, q_end = CEIL_DIV(T, 64);
+    const int q_end = CEIL_DIV(T, 64);
     const int uwave = __builtin_amdgcn_readfirstlane(wave);
     FaLane laq, lado;
     laq.init(lane, uwave, C3);
     lado.init(lane, uwave, (size_t)C);
     base = fa_uniform(base);
     dobase = fa_uniform(dobase);
-    if (q_first < q_end) {
-        fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
-        fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
-    }
-
-    bf16x8 kf[4], vf[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-        if (my_k < T) {
-            kf[s] = *reinterpret_cast<const bf16x8*>(base + C + (size_t)my_k * C3 + 16 * s + 8 * half);
-            vf[s] = *reinterpret_cast<const bf16x8*>(base + 2 * C + (size_t)my_k * C3 + 16 * s + 8 * half);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) { kf[s][e] = (__bf16)0.f; vf[s][e] = (__bf16)0.f; }
+    {
+        const int q_first = (kt_first * 128) / 64;
+        if (q_first < q_end) {
+            fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
+            fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
         }
+        // the per-query statistics of the head go to LDS once (the first tile's queries include the second's): no global
+        // loads besides the tiles inside the loops
+        for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = dbase[q]; }
     }
-    f32x16 dv[2], dk[2];
-#pragma unroll
-    for (int d = 0; d < 2; d++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) { dv[d][r] = 0.f; dk[d][r] = 0.f; }
+    int buf = 0;
 
-    // the per-query statistics of the whole head go to LDS once: no global loads besides the tiles inside the loop
-    for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = dbase[q]; }
-    fa_tiles_landed();
-    __syncthreads();
-
-    for (int qi = q_first; qi < q_end; qi++) {
-        const int buf = (qi - q_first) & 1;
-        const unsigned tq = fa_lds_addr(sQ[buf]), tdo = fa_lds_addr(sdO[buf]);
-        const unsigned stat_l = fa_lds_addr(sLall + 64 * qi), stat_d = fa_lds_addr(sDall + 64 * qi);
-        const bool more = qi + 1 < q_end;
-        if (more) {
-            fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sQ[buf ^ 1]), uwave);
-            fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sdO[buf ^ 1]), uwave);
-        }
+    for (int phase = 0; phase < nphase; phase++) {
+        const int kt = phase == 0 ? kt_first : kt_second;
+        const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
+        const int q_first = (kt * 128) / 64;
+        bf16x8 kf[4], vf[4];
 #pragma unroll
-        for (int qb = 0; qb < 2; qb++) {
-            const int q0 = 64 * qi + 32 * qb;
-            if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
-            f32x16 sacc, pacc;
+        for (int s = 0; s < 4; s++) {
+            if (my_k < T) {
+                kf[s] = *reinterpret_cast<const bf16x8*>(base + C + (size_t)my_k * C3 + 16 * s + 8 * half);
+                vf[s] = *reinterpret_cast<const bf16x8*>(base + 2 * C + (size_t)my_k * C3 + 16 * s + 8 * half);
+            } else {
 #pragma unroll
-            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
-#pragma unroll
-            for (int s = 0; s < 4; s++) {
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
-                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
-            }
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int rr = 32 * qb + g * 8 + half * 4;
-                const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
-            }
-            if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
-#pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int q = q0 + acc_row(r, lane);
-                    if (q < my_k || q >= T) sacc[r] = 0.f;
-                }
-            }
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);     // rowsum(dO*O) of the four queries, read where it is used
-#pragma unroll
-                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[e]);
-            }
-#pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
-#pragma unroll
-                for (int d = 0; d < 2; d++) {
-                    dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
-                    dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tq, laq, 32 * qb + 16 * s2, 32 * d), dsf, dk[d], 0, 0, 0);
-                }
+                for (int e = 0; e < 8; e++) { kf[s][e] = (__bf16)0.f; vf[s][e] = (__bf16)0.f; }
             }
         }
-        fa_tiles_landed();
-        __syncthreads();
-    }
-
-    if (my_k < T) {
-        floatX* dkp = dqkv + ((size_t)b * T + my_k) * C3 + C + h * HS;
-        floatX* dvp = dqkv + ((size_t)b * T + my_k) * C3 + 2 * C + h * HS;
+        f32x16 dv[2], dk[2];
 #pragma unroll
         for (int d = 0; d < 2; d++)
 #pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int col = 32 * d + 8 * g + 4 * half;
-                store4(dkp + col, dk[d][4 * g] * 0.125f, dk[d][4 * g + 1] * 0.125f, dk[d][4 * g + 2] * 0.125f, dk[d][4 * g + 3] * 0.125f);
-                store4(dvp + col, dv[d][4 * g], dv[d][4 * g + 1], dv[d][4 * g + 2], dv[d][4 * g + 3]);
+            for (int r = 0; r < 16; r++) { dv[d][r] = 0.f; dk[d][r] = 0.f; }
+        fa_tiles_landed();                               // the wave's own rows (and, first time, the first tiles and the statistics)
+        if (phase == 0) __syncthreads();
+
+        for (int qi = q_first; qi < q_end; qi++) {
+            const unsigned tq = fa_lds_addr(sQ[buf]), tdo = fa_lds_addr(sdO[buf]);
+            buf ^= 1;
+            const unsigned stat_l = fa_lds_addr(sLall + 64 * qi), stat_d = fa_lds_addr(sDall + 64 * qi);
+            if (qi + 1 < q_end) {
+                fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sQ[buf]), uwave);
+                fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sdO[buf]), uwave);
+            } else if (phase + 1 < nphase) {             // the second tile's first queries
+                const int qn = (kt_second * 128) / 64;
+                fa_tile_request(laq, base + (size_t)(64 * qn) * C3, fa_lds_addr(sQ[buf]), uwave);
+                fa_tile_request(lado, dobase + (size_t)(64 * qn) * C, fa_lds_addr(sdO[buf]), uwave);
             }
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) {
+                const int q0 = 64 * qi + 32 * qb;
+                if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
+                f32x16 sacc, pacc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
+                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int rr = 32 * qb + g * 8 + half * 4;
+                    const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
+                }
+                if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
+#pragma unroll
+                    for (int r = 0; r < 16; r++) {
+                        const int q = q0 + acc_row(r, lane);
+                        if (q < my_k || q >= T) sacc[r] = 0.f;
+                    }
+                }
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);     // rowsum(dO*O) of the four queries, read where it is used
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[e]);
+                }
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++) {
+                    const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
+#pragma unroll
+                    for (int d = 0; d < 2; d++) {
+                        dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
+                        dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tq, laq, 32 * qb + 16 * s2, 32 * d), dsf, dk[d], 0, 0, 0);
+                    }
+                }
+            }
+            fa_tiles_landed();
+            __syncthreads();
+        }
+
+        if (my_k < T) {
+            floatX* dkp = dqkv + ((size_t)b * T + my_k) * C3 + C + h * HS;
+            floatX* dvp = dqkv + ((size_t)b * T + my_k) * C3 + 2 * C + h * HS;
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int col = 32 * d + 8 * g + 4 * half;
+                    store4(dkp + col, dk[d][4 * g] * 0.125f, dk[d][4 * g + 1] * 0.125f, dk[d][4 * g + 2] * 0.125f, dk[d][4 * g + 3] * 0.125f);
+                    store4(dvp + col, dv[d][4 * g], dv[d][4 * g + 1], dv[d][4 * g + 2], dv[d][4 * g + 3]);
+                }
+        }
     }
 }
 
@@ -883,13 +913,16 @@ fa_backward_dq_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout
 // which takes the place of fa_dot_do_o_kernel's pass over dO and O: it runs before the dK/dV kernel.
 __global__ void __launch_bounds__(256, 4)
 fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
-                          const floatX* __restrict__ o, const float* __restrict__ stats, float* __restrict__ Dsum, int T, int NH) {
+                          const floatX* __restrict__ o, const float* __restrict__ stats, float* __restrict__ Dsum, int T, int NH,
+                          int nq) {
     __shared__ __attribute__((aligned(1024))) char sK[2][SW_TILE];
     __shared__ __attribute__((aligned(1024))) char sV[2][SW_TILE];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
     int tile_x, bh;
     fa_block_coords(tile_x, bh);
-    const int qt = gridDim.x - 1 - tile_x;
+    // two query tiles per workgroup, nq - 1 - x and then x, as in fa_forward_dma_kernel: equal work for every workgroup
+    const int qt_first = nq - 1 - tile_x, qt_second = tile_x;
+    const int nphase = qt_first == qt_second ? 1 : 2;
     const int b = bh / NH, h = bh % NH;
     const int C = NH * HS;
     const size_t C3 = 3 * (size_t)C;
@@ -902,91 +935,99 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
     const floatX* vbase = fa_uniform(base + 2 * C);
     fa_tile_request(la, kbase, fa_lds_addr(sK[0]), uwave);
     fa_tile_request(la, vbase, fa_lds_addr(sV[0]), uwave);
-    const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
     const float c = 0.125f * LOG2E;
+    int buf = 0;
 
-    bf16x8 qf[4], dof[4];
-#pragma unroll
-    for (int s = 0; s < 4; s++) {
-        if (my_q < T) {
-            qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
-            dof[s] = *reinterpret_cast<const bf16x8*>(dout + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
-        } else {
-#pragma unroll
-            for (int e = 0; e < 8; e++) { qf[s][e] = (__bf16)0.f; dof[s][e] = (__bf16)0.f; }
-        }
-    }
-    const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
-    // D = rowsum(dO * O) of the lane's query from the dO values it already holds: the two halves of the wave own
-    // 32 head dimensions each. The dK/dV kernel, launched after this one, reads D from memory.
-    float dsum = 0.f;
-    if (my_q < T) {
+    for (int phase = 0; phase < nphase; phase++) {
+        const int qt = phase == 0 ? qt_first : qt_second;
+        const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+        bf16x8 qf[4], dof[4];
 #pragma unroll
         for (int s = 0; s < 4; s++) {
-            const bf16x8 of = *reinterpret_cast<const bf16x8*>(o + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
+            if (my_q < T) {
+                qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
+                dof[s] = *reinterpret_cast<const bf16x8*>(dout + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
+            } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) dsum = fmaf((float)dof[s][e], (float)of[e], dsum);
+                for (int e = 0; e < 8; e++) { qf[s][e] = (__bf16)0.f; dof[s][e] = (__bf16)0.f; }
+            }
         }
-    }
-    dsum += __shfl_xor(dsum, 32, WAVE);
-    if (my_q < T && half == 0) Dsum[((size_t)b * NH + h) * T + my_q] = dsum;
-    f32x16 dq[2];
-#pragma unroll
-    for (int d = 0; d < 2; d++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) dq[d][r] = 0.f;
-
-    const int last_q = min(qt * 128 + 127, T - 1);
-    const int n_kt = last_q / 64 + 1;
-    fa_tiles_landed();
-    __syncthreads();
-
-    for (int j = 0; j < n_kt; j++) {
-        const unsigned tk = fa_lds_addr(sK[j & 1]), tv = fa_lds_addr(sV[j & 1]);
-        if (j + 1 < n_kt) {                              // the other buffer was last read before the barrier that ended step j - 1
-            fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[(j + 1) & 1]), uwave);
-            fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[(j + 1) & 1]), uwave);
-        }
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            const int k0 = 64 * j + 32 * kb;
-            if (k0 > qw0 + 31) continue;
-            f32x16 sacc, pacc;
-#pragma unroll
-            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+        const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
+        // D = rowsum(dO * O) of the lane's query from the dO values it already holds: the two halves of the wave own
+        // 32 head dimensions each. The dK/dV kernel, launched after this one, reads D from memory.
+        float dsum = 0.f;
+        if (my_q < T) {
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
-                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
-            }
+                const bf16x8 of = *reinterpret_cast<const bf16x8*>(o + ((size_t)b * T + my_q) * C + h * HS + 16 * s + 8 * half);
 #pragma unroll
-            for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
-            if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
-#pragma unroll
-                for (int r = 0; r < 16; r++)
-                    if (k0 + acc_row(r, lane) > my_q) sacc[r] = 0.f;
-            }
-#pragma unroll
-            for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
-#pragma unroll
-            for (int s2 = 0; s2 < 2; s2++) {
-                const bf16x8 dsf = pack_acc(pacc, s2);
-#pragma unroll
-                for (int d = 0; d < 2; d++)
-                    dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
+                for (int e = 0; e < 8; e++) dsum = fmaf((float)dof[s][e], (float)of[e], dsum);
             }
         }
-        fa_tiles_landed();
-        __syncthreads();
-    }
-    if (my_q < T) {
-        floatX* dqp = dqkv + ((size_t)b * T + my_q) * C3 + h * HS;
+        dsum += __shfl_xor(dsum, 32, WAVE);
+        if (my_q < T && half == 0) Dsum[((size_t)b * NH + h) * T + my_q] = dsum;
+        f32x16 dq[2];
 #pragma unroll
         for (int d = 0; d < 2; d++)
 #pragma unroll
-            for (int g = 0; g < 4; g++)
-                store4(dqp + 32 * d + 8 * g + 4 * half, dq[d][4 * g] * 0.125f, dq[d][4 * g + 1] * 0.125f, dq[d][4 * g + 2] * 0.125f,
-                       dq[d][4 * g + 3] * 0.125f);
+            for (int r = 0; r < 16; r++) dq[d][r] = 0.f;
+
+        const int last_q = min(qt * 128 + 127, T - 1);
+        const int n_kt = last_q / 64 + 1;
+        fa_tiles_landed();                               // the wave's own rows (and the first keys of the first tile)
+        if (phase == 0) __syncthreads();
+
+        for (int j = 0; j < n_kt; j++) {
+            const unsigned tk = fa_lds_addr(sK[buf]), tv = fa_lds_addr(sV[buf]);
+            buf ^= 1;
+            if (j + 1 < n_kt) {                          // the other buffer was last read before the barrier that ended the previous step
+                fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[buf]), uwave);
+                fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[buf]), uwave);
+            } else if (phase + 1 < nphase) {             // the second tile starts over at the head's first keys
+                fa_tile_request(la, kbase, fa_lds_addr(sK[buf]), uwave);
+                fa_tile_request(la, vbase, fa_lds_addr(sV[buf]), uwave);
+            }
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+                const int k0 = 64 * j + 32 * kb;
+                if (k0 > qw0 + 31) continue;
+                f32x16 sacc, pacc;
+#pragma unroll
+                for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+#pragma unroll
+                for (int s = 0; s < 4; s++) {
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
+                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
+                if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
+#pragma unroll
+                    for (int r = 0; r < 16; r++)
+                        if (k0 + acc_row(r, lane) > my_q) sacc[r] = 0.f;
+                }
+#pragma unroll
+                for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
+#pragma unroll
+                for (int s2 = 0; s2 < 2; s2++) {
+                    const bf16x8 dsf = pack_acc(pacc, s2);
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+                        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
+                }
+            }
+            fa_tiles_landed();
+            __syncthreads();
+        }
+        if (my_q < T) {
+            floatX* dqp = dqkv + ((size_t)b * T + my_q) * C3 + h * HS;
+#pragma unroll
+            for (int d = 0; d < 2; d++)
+#pragma unroll
+                for (int g = 0; g < 4; g++)
+                    store4(dqp + 32 * d + 8 * g + 4 * half, dq[d][4 * g] * 0.125f, dq[d][4 * g + 1] * 0.125f, dq[d][4 * g + 2] * 0.125f,
+                           dq[d][4 * g + 3] * 0.125f);
+        }
     }
 }
 
@@ -1208,12 +1249,16 @@ void attention_backward_impl(void* dqkvr, const void* dout, const void* qkvr, co
         if (T % 64 == 0) {                      // whole tiles only: direct-to-LDS kernels, dQ first (it also leaves D for dK/dV)
             {
                 llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dq", 1.0 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
-                fa_backward_dq_dma_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH);
+                const int nq = CEIL_DIV(T, 128);             // a workgroup takes two query tiles
+                fa_backward_dq_dma_kernel<<<dim3((nq + 1) / 2, B * NH), 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, (const floatX*)o, stats, Dsum, T, NH, nq);
                 LAUNCH_CHECK();
             }
             llmk::ProfScope prof(Dsum_static != nullptr, "attention_backward_dkdv", 1.5 * fwd_flops, 6.0 * B * T * C * sizeof(floatX), st);
             if (T <= 4096)                      // 2*T floats of statistics in LDS beside the 32 KiB of tiles
-                fa_backward_dkdv_dma_kernel<<<grid, 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
+            {
+                const int nk = CEIL_DIV(T, 128);             // a workgroup takes two key tiles
+                fa_backward_dkdv_dma_kernel<<<dim3((nk + 1) / 2, B * NH), 256, 2 * (size_t)T * sizeof(float), st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH, nk);
+            }
             else
                 fa_backward_dkdv_kernel<<<grid, 256, 0, st>>>((floatX*)dqkvr, (const floatX*)dout, (const floatX*)qkvr, stats, Dsum, T, NH);
             LAUNCH_CHECK();
@@ -1261,7 +1306,10 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
     if (hs == HS) {
         LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
         if (T % 64 == 0)
-            fa_forward_dma_kernel<<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
+        {
+            const int nq = CEIL_DIV(T, 128);                 // query tiles of a head; a workgroup takes two of them
+            fa_forward_dma_kernel<<<dim3((nq + 1) / 2, B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH, nq);
+        }
         else
             fa_forward_kernel<4><<<dim3(CEIL_DIV(T, 128), B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH);
         LAUNCH_CHECK();
