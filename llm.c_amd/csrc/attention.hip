@@ -105,7 +105,9 @@ __device__ __forceinline__ void store4(floatX* p, float a, float b, float c, flo
 // side (lane p of a row fetches chunk p ^ swz(row)). swz is chosen so that 16 consecutive rows read at one chunk
 // (MFMA operand along rows) and 4 rows x 32 B (transposing reads) both spread over all banks.
 constexpr int SW_TILE = 64 * 128;
-__device__ __forceinline__ int fa_swz(int row) { return (((row >> 1) & 3) << 1) | ((row >> 3) & 1); }
+// swz = the three bits of row >> 1 in reverse order: rows 2 apart (the ones a transposing read takes from the same half
+// of the banks in one cycle) land 64 bytes apart, and the 8 even (odd) rows of a 16-row column read get 8 different chunks.
+__device__ __forceinline__ int fa_swz(int row) { return (((row >> 1) & 1) << 2) | (((row >> 2) & 1) << 1) | ((row >> 3) & 1); }
 typedef __attribute__((address_space(3))) void* fa_lds_ptr;
 struct FaLane {
     unsigned rowb;          // frag along rows: byte offset of (row = lane%32, K step 0); step s is rowb ^ (s << 5)
