@@ -66,6 +66,13 @@ __device__ __forceinline__ bf16x8 pack_acc(const f32x16& a, int s2) {
     for (int e = 0; e < 8; e++) o[e] = (__bf16)a[8 * s2 + e];
     return o;
 }
+// The lane id as a value the compiler cannot trace back: what is derived from it (row offsets, per-lane pointers) is then
+// formed where it is used and dies there, instead of being carried in registers through the tile loops of kernels that
+// have none to spare.
+__device__ __forceinline__ int fresh_lane(int lane) {
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
 // row index (within a 32-row block) of accumulator register r for this lane
 __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
 
@@ -164,6 +171,14 @@ __device__ __forceinline__ unsigned fa_lds_addr(const void* p) {
 __device__ __forceinline__ bf16x8 fa_frag_rows(unsigned tile, const FaLane& a, int row0, int s) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)(tile + row0 * 128 + (a.rowb ^ (unsigned)(s << 5))));
 }
+// A value the compiler must take as new at this point: what is derived from it is computed here, next to its use,
+// instead of once before the loop and kept in a register of its own for the whole kernel.
+__device__ __forceinline__ unsigned fa_fresh(unsigned v) { asm volatile("" : "+v"(v)); return v; }
+// The same reads for a kernel short of registers: the swizzled address of each step is formed at the read (one
+// xor-add) rather than held for the life of the kernel.
+__device__ __forceinline__ bf16x8 fa_frag_rows_lean(unsigned tile, const FaLane& a, int row0, int s) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)((fa_fresh(a.rowb) ^ (unsigned)(s << 5)) + (tile + row0 * 128)));
+}
 __device__ __forceinline__ f32x4 fa_lds_f32x4(unsigned addr) {
     return *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>((size_t)addr);
 }
@@ -173,6 +188,16 @@ __device__ __forceinline__ bf16x8 fa_frag_cols(unsigned tile, const FaLane& a, i
     const unsigned x = col0 ? 64u : 0u, t = tile + kbase * 128;
     s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(t + (a.colb0 ^ x)));
     s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(t + (a.colb1 ^ x)));
+    union { struct { s16x4 a, b; } s; bf16x8 v; } u;
+    u.s.a = lo; u.s.b = hi;
+    return u.v;
+}
+
+__device__ __forceinline__ bf16x8 fa_frag_cols_lean(unsigned tile, const FaLane& a, int kbase, int col0) {
+    typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
+    const unsigned x = col0 ? 64u : 0u, t = tile + kbase * 128;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)((fa_fresh(a.colb0) ^ x) + t));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)((fa_fresh(a.colb1) ^ x) + t));
     union { struct { s16x4 a, b; } s; bf16x8 v; } u;
     u.s.a = lo; u.s.b = hi;
     return u.v;
@@ -401,14 +426,17 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
 
     for (int phase = 0; phase < nphase; phase++) {
         const int qt = phase == 0 ? qt_first : qt_second;
-        const int qw0 = qt * GQ + wave * 32, my_q = qw0 + idx;
+        const int qw0 = qt * GQ + uwave * 32;             // wave-uniform
         bf16x8 qf[4];
+        {
+            const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_q = qw0 + idx;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             if (my_q < T) qf[s] = *reinterpret_cast<const bf16x8*>(base + (size_t)my_q * C3 + 16 * s + 8 * half);
             else
 #pragma unroll
                 for (int e = 0; e < 8; e++) qf[s][e] = (__bf16)0.f;
+        }
         }
         f32x16 o[2];
 #pragma unroll
@@ -452,11 +480,14 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
                 }
                 if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
                     asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
+                    // key 64j + 32kb + acc_row(r) against query qw0 + idx: the lane's share of both sides is one small number
+                    const int ln = fresh_lane(lane);
+                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = qw0 - 64 * j;
 #pragma unroll
                     for (int kb = 0; kb < 2; kb++)
 #pragma unroll
                         for (int r = 0; r < 16; r++)
-                            if (64 * j + 32 * kb + acc_row(r, lane) > my_q) sacc[kb][r] = -INFINITY;
+                            if (32 * kb + (r >> 2) * 8 + (r & 3) + dl > lim) sacc[kb][r] = -INFINITY;
                 }
                 float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
@@ -496,6 +527,7 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
         }
 
         const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
+        const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_q = qw0 + idx;
         if (my_q < T) {
             const float inv = 1.0f / l;
             floatX* dst = out + ((size_t)b * T + my_q) * C + h * HS;
@@ -716,9 +748,11 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
 
     for (int phase = 0; phase < nphase; phase++) {
         const int kt = phase == 0 ? kt_first : kt_second;
-        const int kw0 = kt * 128 + wave * 32, my_k = kw0 + idx;
+        const int kw0 = kt * 128 + uwave * 32;           // wave-uniform
         const int q_first = (kt * 128) / 64;
         bf16x8 kf[4], vf[4];
+        {
+        const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_k = kw0 + idx;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             if (my_k < T) {
@@ -728,6 +762,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
 #pragma unroll
                 for (int e = 0; e < 8; e++) { kf[s][e] = (__bf16)0.f; vf[s][e] = (__bf16)0.f; }
             }
+        }
         }
         f32x16 dv[2], dk[2];
 #pragma unroll
@@ -769,9 +804,10 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                     for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
                 }
                 if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
+                    const int ln = fresh_lane(lane), my_k = kw0 + (ln & 31);
 #pragma unroll
                     for (int r = 0; r < 16; r++) {
-                        const int q = q0 + acc_row(r, lane);
+                        const int q = q0 + acc_row(r, ln);
                         if (q < my_k || q >= T) sacc[r] = 0.f;
                     }
                 }
@@ -795,6 +831,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
             __syncthreads();
         }
 
+        const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_k = kw0 + idx;
         if (my_k < T) {
             floatX* dkp = dqkv + ((size_t)b * T + my_k) * C3 + C + h * HS;
             floatX* dvp = dqkv + ((size_t)b * T + my_k) * C3 + 2 * C + h * HS;
@@ -942,8 +979,11 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
 
     for (int phase = 0; phase < nphase; phase++) {
         const int qt = phase == 0 ? qt_first : qt_second;
-        const int qw0 = qt * 128 + wave * 32, my_q = qw0 + idx;
+        const int qw0 = qt * 128 + uwave * 32;           // wave-uniform
         bf16x8 qf[4], dof[4];
+        float lse2, dsum = 0.f;
+        {
+        const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_q = qw0 + idx;
 #pragma unroll
         for (int s = 0; s < 4; s++) {
             if (my_q < T) {
@@ -954,10 +994,9 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
                 for (int e = 0; e < 8; e++) { qf[s][e] = (__bf16)0.f; dof[s][e] = (__bf16)0.f; }
             }
         }
-        const float lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
+        lse2 = my_q < T ? stats[((size_t)b * NH + h) * T + my_q] * LOG2E : 0.f;
         // D = rowsum(dO * O) of the lane's query from the dO values it already holds: the two halves of the wave own
         // 32 head dimensions each. The dK/dV kernel, launched after this one, reads D from memory.
-        float dsum = 0.f;
         if (my_q < T) {
 #pragma unroll
             for (int s = 0; s < 4; s++) {
@@ -968,6 +1007,7 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
         }
         dsum += __shfl_xor(dsum, 32, WAVE);
         if (my_q < T && half == 0) Dsum[((size_t)b * NH + h) * T + my_q] = dsum;
+        }
         f32x16 dq[2];
 #pragma unroll
         for (int d = 0; d < 2; d++)
@@ -997,16 +1037,19 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
 #pragma unroll
                 for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
 #pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
-                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
-                }
+                for (int s = 0; s < 4; s++)
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
                 if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
+                    const int ln = fresh_lane(lane);
+                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = qw0 - k0;      // key k0 + acc_row(r) against query qw0 + idx
 #pragma unroll
                     for (int r = 0; r < 16; r++)
-                        if (k0 + acc_row(r, lane) > my_q) sacc[r] = 0.f;
+                        if ((r >> 2) * 8 + (r & 3) + dl > lim) sacc[r] = 0.f;
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
@@ -1015,12 +1058,13 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
                     const bf16x8 dsf = pack_acc(pacc, s2);
 #pragma unroll
                     for (int d = 0; d < 2; d++)
-                        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
+                        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols_lean(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
                 }
             }
             fa_tiles_landed();
             __syncthreads();
         }
+        const int ln = fresh_lane(lane), idx = ln & 31, half = ln >> 5, my_q = qw0 + idx;
         if (my_q < T) {
             floatX* dqp = dqkv + ((size_t)b * T + my_q) * C3 + h * HS;
 #pragma unroll
