@@ -342,8 +342,10 @@ def main():
     if default_headline(args) and not args.no_other_configs:
         # BASELINE configs[3] and configs[4], a few steps each, after and outside the headline measurement
         out["other_configs"] = []
-        for model, b, lr in (("d24", 32, 3e-4), ("d48", 16, 6e-4)):          # learning rates of the reference's recipes
-            r = run_workload(L, torch, model, b, 1024, 1, 2, 3, 1, False, lr=lr)
+        # batch, recompute setting and learning rate of the reference's recipes (scripts/run_gpt2_350M.sh:29-34,
+        # scripts/run_gpt2_1558M.sh:27-33: -b 64 / -b 16, -r 0)
+        for model, b, lr in (("d24", 64, 3e-4), ("d48", 16, 6e-4)):
+            r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 1, False, lr=lr)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
                                                               "loss_first", "loss_last")})
     if not args.no_cpu_baseline:
