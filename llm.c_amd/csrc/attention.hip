@@ -19,6 +19,7 @@
 // fp32 build: straightforward one-wave-per-row kernels (lanes = head dimensions), used only for
 // parity runs against the CPU reference at small sizes.
 #include "common.hpp"
+#include <type_traits>
 #include "../../include/llmk.h"
 
 namespace {
@@ -387,7 +388,8 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
     }
 }
 
-// The same forward pass with K and V brought in by direct-to-LDS loads (T a multiple of 64: every tile is whole).
+// The same forward pass with K and V brought in by direct-to-LDS loads (T a multiple of 128: every tile is whole and a
+// query tile walks an even number of key tiles).
 // Without the staging registers the kernel fits 128 VGPRs, a fourth wave per SIMD, and with the loads issued from
 // inline asm the reads of the tile in use do not wait for the tile in flight. Same arithmetic in the same order as
 // fa_forward_kernel: the two give identical bits.
@@ -422,7 +424,6 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
     bf16x8 ones;
 #pragma unroll
     for (int e = 0; e < 8; e++) ones[e] = (__bf16)1.0f;
-    int buf = 0;                                          // the buffer that holds the key tile of the coming step
 
     for (int phase = 0; phase < nphase; phase++) {
         const int qt = phase == 0 ? qt_first : qt_second;
@@ -456,9 +457,12 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
         fa_tiles_landed();
         if (phase == 0) __syncthreads();
 
-        for (int j = 0; j < n_kt; j++) {
-            const unsigned tk = fa_lds_addr(sK[buf]), tv = fa_lds_addr(sV[buf]);
-            buf ^= 1;
+        // One step = one tile of 64 keys. The buffer is a compile-time constant (the loop below alternates two copies of
+        // the step), so a fragment's LDS address is a lane register plus an immediate: no vector add per read.
+        auto step = [&](int j, auto bufc) {
+            constexpr int BUF = decltype(bufc)::value;
+            const unsigned tk = fa_lds_addr(sK[BUF]), tv = fa_lds_addr(sV[BUF]);
+            constexpr int buf = BUF ^ 1;
             if (j + 1 < n_kt) {                          // the other buffer was last read before the barrier that ended the previous step
                 fa_tile_request(la, kbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sK[buf]), uwave);
                 fa_tile_request(la, vbase + (size_t)(64 * (j + 1)) * C3, fa_lds_addr(sV[buf]), uwave);
@@ -524,6 +528,10 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
             }
             fa_tiles_landed();
             __syncthreads();
+        };
+        for (int j = 0; j < n_kt; j += 2) {             // n_kt is even: a tile of 128 queries ends on a multiple of 128 keys
+            step(j, std::integral_constant<int, 0>{});
+            step(j + 1, std::integral_constant<int, 1>{});
         }
 
         const float l = lacc[0];                              // complete: the MFMA already summed over all 32 keys of both halves
@@ -1351,7 +1359,7 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
 #if !defined(LLMK_FP32)
     if (hs == HS) {
         LLMK_REQUIRE(((uintptr_t)inp % 16) == 0 && ((uintptr_t)out % 8) == 0, "attention_forward: misaligned buffers");
-        if (T % 64 == 0)
+        if (T % 128 == 0)                       // whole tiles of 128 queries: an even number of key tiles per query tile
         {
             const int nq = CEIL_DIV(T, 128);                 // query tiles of a head; a workgroup takes two of them
             fa_forward_dma_kernel<<<dim3((nq + 1) / 2, B * NH), 256, 0, st>>>((floatX*)out, stats, (const floatX*)inp, T, NH, nq);
