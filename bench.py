@@ -260,7 +260,7 @@ def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, k
                    "global_batch": B, "seq_len": T, "tokens_per_step": B * T, "recompute": recompute,
                    "gelu_fusion": gelu_fusion, "parallelism": "single GPU"},
         "mfu": float(mfu), "mfu_peak_tflops": PEAK_BF16_TFLOPS,
-        "loss_first": float(losses[0]), "loss_last": float(losses[-1]),
+        "loss_first": float(losses[0]), "loss_last": float(losses[-1]), "losses": [round(float(x), 4) for x in losses],
         "roofline": roofline, "kernels_from_last_warmup_step": kernels,
     }
 
@@ -345,9 +345,9 @@ def main():
         # batch, recompute setting and learning rate of the reference's recipes (scripts/run_gpt2_350M.sh:29-34,
         # scripts/run_gpt2_1558M.sh:27-33: -b 64 / -b 16, -r 0)
         for model, b, lr in (("d24", 64, 3e-4), ("d48", 16, 6e-4)):
-            r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 1, False, lr=lr)
+            r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 2, False, lr=lr)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
-                                                              "loss_first", "loss_last")})
+                                                              "loss_first", "loss_last", "losses")})
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     C.CDLL(None).fflush(None)
