@@ -4,6 +4,7 @@
 // 64-wide wavefronts.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <type_traits>
 #include <hip/hip_bf16.h>
 #include <cstdint>
 #include <cstdio>
@@ -129,6 +130,23 @@ __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, WAVE);
     return v;
+}
+// The same sum through the data-parallel-primitive lane moves of the vector ALU instead of six trips through the LDS
+// crossbar: prefix sums inside each row of 16 lanes, row totals passed on to the later rows, lane 63's total read
+// back as a wave-uniform value. A different (fixed) summation order than wave_sum's butterfly.
+__device__ __forceinline__ float wave_sum_dpp(float v) {
+    auto shifted = [](float x, auto ctrl, auto row_mask) -> float {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), decltype(ctrl)::value,
+                                                                     decltype(row_mask)::value, 0xf, true));
+    };
+    using std::integral_constant;
+    v += shifted(v, integral_constant<int, 0x111>{}, integral_constant<int, 0xf>{});     // row_shr:1
+    v += shifted(v, integral_constant<int, 0x112>{}, integral_constant<int, 0xf>{});     // row_shr:2
+    v += shifted(v, integral_constant<int, 0x114>{}, integral_constant<int, 0xf>{});     // row_shr:4
+    v += shifted(v, integral_constant<int, 0x118>{}, integral_constant<int, 0xf>{});     // row_shr:8: lane 15 of a row has the row's sum
+    v += shifted(v, integral_constant<int, 0x142>{}, integral_constant<int, 0xa>{});     // row_bcast:15 into rows 1 and 3
+    v += shifted(v, integral_constant<int, 0x143>{}, integral_constant<int, 0xc>{});     // row_bcast:31 into rows 2 and 3
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 __device__ __forceinline__ float wave_max(float v) {
 #pragma unroll
