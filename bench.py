@@ -340,11 +340,12 @@ def main():
         out["sclk_mhz_during_timed_steps"] = step_clock.median()
 
     if default_headline(args) and not args.no_other_configs:
-        # BASELINE configs[3] and configs[4], a few steps each, after and outside the headline measurement
+        # a few steps each of the larger configurations, after and outside the headline measurement
         out["other_configs"] = []
-        # batch, recompute setting and learning rate of the reference's recipes (scripts/run_gpt2_350M.sh:29-34,
-        # scripts/run_gpt2_1558M.sh:27-33: -b 64 / -b 16, -r 0)
-        for model, b, lr in (("d24", 64, 3e-4), ("d48", 16, 6e-4)):
+        # BASELINE configs[3] (350M, B=32) and configs[4] (1558M, B=16), then the 350M model at the batch of the reference's
+        # own recipe (scripts/run_gpt2_350M.sh:29-34: -b 64; scripts/run_gpt2_1558M.sh:27-33 has -b 16). No recomputation
+        # (-r 0) and the learning rates of those recipes.
+        for model, b, lr in (("d24", 32, 3e-4), ("d48", 16, 6e-4), ("d24", 64, 3e-4)):
             r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 2, False, lr=lr)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
                                                               "loss_first", "loss_last", "losses")})
