@@ -133,6 +133,13 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                           const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
                           const void* pre_gelu, int gelu_fusion);
 size_t llmk_matmul_backward_bias_scratch_floats(int OC);
+/* How llmk_matmul_backward cuts the weight gradient's contraction over B*T into work items (bf16 library): -1 (default)
+ * picks by a cost estimate between equal splits of every tile and, when the tiles are a sizable part of the workgroups
+ * of a launch, one long and a few short pieces per tile (cut at the same K positions for every tile, scheduled so that
+ * all workgroups finish together); 0 always takes equal splits, 1 takes the uneven pieces whenever the shape allows
+ * them. The result is the same sum in a different (fixed) order of fp32 partials. No counterpart in the reference
+ * (cuBLASLt chooses its own split there); for tests and tuning. */
+void llmk_matmul_backward_split_mode(int mode);
 
 /* gelu_backward_inplace (llmc/gelu.cuh:59) and the bias gradient of matmul_backward (llmc/matmul.cuh:251-266) in
  * one pass over (B*T, OC): d_in_out *= gelu'(inp), then dbias[OC] += column sums of the result. Same values as

@@ -41,6 +41,7 @@ KERNEL_ABI = {
     "llmk_last_error": (C.c_char_p, []),
     "llmk_clear_error": (None, []),
     "llmk_profile_enable": (None, [i32]),
+    "llmk_matmul_backward_split_mode": (None, [i32]),
     "llmk_profile_only": (None, [C.c_char_p]),
     "llmk_zero": (None, [vp, C.c_size_t, vp]),
     "llmk_probe_mfma_peak": (None, [C.POINTER(C.c_double), vp, vp]),

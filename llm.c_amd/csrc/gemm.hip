@@ -27,6 +27,8 @@
 #include "common.hpp"
 #include "gelu.hpp"
 #include "gemm_pipelined.hpp"
+#include <vector>
+#include <algorithm>
 #include "../../include/llmk.h"
 
 namespace {
@@ -465,6 +467,82 @@ splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, 
     }
 }
 
+#if !defined(LLMK_FP32)
+// Cutting the weight gradient's contraction when its T tiles are a sizable part of the G workgroups (GPT-2 1558M at B*T =
+// 16384: 133-175 tiles of 256 x 256 for 256 CUs). Equal splits fill the launch only at 4-5 per tile, and each split costs a
+// pass of fp32 partials over the output. Here every tile is cut at the SAME K positions into one long piece and s - 1
+// short ones: T workgroups take a long piece each, the other G - T take p short pieces each, and the cut is placed where
+// both finish together (long = p x short). The pieces that run side by side still cover the same K range, so the 32 CUs
+// of an XCD go on sharing operand panels through their L2 (handing out contiguous (tile, K) ranges of equal length
+// instead, each workgroup at its own K offset, left every panel to be streamed once per tile: slower than the equal
+// splits). Partial slot = rank of the piece along K, so the sum order is fixed.
+constexpr int SK_MIN_BLOCKS = 4;
+int g_sk_mode = -1;                  // llmk_matmul_backward_split_mode
+struct SkPlan {
+    int tiles_m = 0, tiles_n = 0, kblocks = 0, G = 0;
+    int slots = 0;                   // pieces per tile
+    double cost = 1e30;              // launch time in units of the perfectly balanced GEMM, partial passes included
+    unsigned* d_items = nullptr;     // [G][SK_MAX_ITEMS][2]
+    std::vector<unsigned> items;
+    bool valid = false, uploaded = false;
+};
+void sk_build(SkPlan& p, int tiles_m, int tiles_n, int kblocks, int G, double pass) {
+    p.tiles_m = tiles_m; p.tiles_n = tiles_n; p.kblocks = kblocks; p.G = G; p.valid = false;
+    const int T = tiles_m * tiles_n, S = kblocks;
+    if (tiles_m >= 4096 || tiles_n >= 4096 || S >= 65536 || T >= G || T * 8 < G) return;
+    int best_s = 0, best_x = 0, best_p = 0;
+    for (int s = 2; s <= 6; s++) {
+        const int ny = T * (s - 1), p_each = CEIL_DIV(ny, G - T);
+        if (p_each + 1 > SK_MAX_ITEMS) continue;
+        int x = (int)((long long)p_each * S / (s - 1 + p_each));           // long piece = p short ones
+        const int y_max = CEIL_DIV(S - x, s - 1), y_min = (S - x) / (s - 1);
+        if (x < SK_MIN_BLOCKS || y_min < SK_MIN_BLOCKS) continue;
+        const int makespan = std::max(x, p_each * y_max);
+        const double cost = (double)makespan * G / ((double)T * S) + pass * s;
+        if (cost < p.cost) { p.cost = cost; best_s = s; best_x = x; best_p = p_each; }
+    }
+    if (!best_s) return;
+    const int s = best_s, x = best_x;
+    p.slots = s;
+    p.items.assign((size_t)G * SK_MAX_ITEMS * 2, 0u);
+    auto put = [&](int c, int n, int t, int slot, int k0, int len) {
+        const unsigned tm = (unsigned)(t / tiles_n), tn = (unsigned)(t % tiles_n);
+        p.items[((size_t)c * SK_MAX_ITEMS + n) * 2] = tm | (tn << 12) | ((unsigned)slot << 24);
+        p.items[((size_t)c * SK_MAX_ITEMS + n) * 2 + 1] = (unsigned)k0 | ((unsigned)len << 16);
+    };
+    for (int t = 0; t < T; t++) put(t, 0, t, 0, 0, x);                      // list t: the long piece of tile t
+    // the short pieces in (K range, tile) order, best_p at a time to the remaining lists
+    int c = T, n = 0;
+    for (int j = 1; j < s; j++) {
+        const int k0 = x + (int)((long long)(S - x) * (j - 1) / (s - 1)), k1 = x + (int)((long long)(S - x) * j / (s - 1));
+        for (int t = 0; t < T; t++) {
+            if (n == best_p) { c++; n = 0; }
+            if (c >= G) return;                                            // cannot happen: (G - T) * best_p >= T * (s - 1)
+            put(c, n++, t, j, k0, k1 - k0);
+        }
+    }
+    p.valid = true;
+}
+// plans are kept for the life of the process (a training run has four to six shapes), their device copies with them
+SkPlan* sk_plan(int tiles_m, int tiles_n, int kblocks, int G, double pass) {
+    static std::vector<SkPlan*> plans;
+    for (SkPlan* q : plans)
+        if (q->tiles_m == tiles_m && q->tiles_n == tiles_n && q->kblocks == kblocks && q->G == G) return q;
+    SkPlan* p = new SkPlan();
+    sk_build(*p, tiles_m, tiles_n, kblocks, G, pass);
+    plans.push_back(p);
+    return p;
+}
+bool sk_upload(SkPlan& p) {
+    if (p.uploaded) return true;
+    if (hipMalloc(&p.d_items, p.items.size() * sizeof(unsigned)) != hipSuccess) return false;
+    // a synchronous copy, once per shape
+    if (hipMemcpy(p.d_items, p.items.data(), p.items.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess) return false;
+    p.uploaded = true;
+    return true;
+}
+#endif
+
 // ---- bias gradient: column sums of dout[N][OC] -----------------------------------------------
 // HBM-bound streaming reduction. Workgroup = 32 column-vectors (512 B of a row) x 8 row lanes; each lane keeps
 // four row loads in flight. grid.y splits the rows so that ~2 workgroups per CU are resident; their partial sums
@@ -667,6 +745,14 @@ void llmk_gelu_backward_bias(void* d_in_out, const void* inp, void* dbias, float
 
 size_t llmk_matmul_backward_bias_scratch_floats(int OC) { return (size_t)bias_grad_ny(OC) * OC; }
 
+void llmk_matmul_backward_split_mode(int mode) {
+#if !defined(LLMK_FP32)
+    g_sk_mode = mode < 0 ? -1 : mode > 0 ? 1 : 0;
+#else
+    (void)mode;                          // the fp32 library has one weight-gradient path
+#endif
+}
+
 void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
                           const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
                           const void* pre_gelu, int gelu_fusion) {
@@ -757,6 +843,11 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                 if (cost < best) { best = cost; splits = s; }
             }
         }
+        double best_uniform = 1e30;
+        {
+            const size_t work = tiles * splits, rounds = CEIL_DIV(work, (size_t)num_cu);
+            best_uniform = (double)(rounds * num_cu) / (double)work + 800.0 / (double)M * splits;
+        }
         const int ksteps = CEIL_DIV(M, K_STEP);
         splits = min(splits, max(1, ksteps / 8));                 // at least 8 K steps per split
         const int steps_per = CEIL_DIV(ksteps, splits);
@@ -767,6 +858,42 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
             LLMK_REQUIRE(!dbias_in_gemm, "matmul_backward: bias gradient was left to a kernel that is not being run");
             llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
             launch_best<true, true, EPI_ACCUM>(g, 1, big, st);
+#if !defined(LLMK_FP32)
+        } else if (SkPlan* plan = (big && M % K_STEP == 0 && pipelined_ok(g) && (!dbias || dbias_in_gemm) && g_sk_mode != 0)
+                                      ? sk_plan(CEIL_DIV(OC, BIG_TILE), CEIL_DIV(C, BIG_TILE), M / K_STEP, num_cu & ~7, 800.0 / (double)M)
+                                      : nullptr;
+                   plan && plan->valid && (g_sk_mode == 1 || plan->cost < 0.98 * best_uniform) && sk_upload(*plan)) {
+            // one long and s - 1 short pieces per tile, scheduled by the host's list (see sk_build)
+            const size_t mn = (size_t)OC * C;
+            const int parts = 4, slots = plan->slots;
+            g.partial = (float*)llmk::workspace((mn + (dbias_in_gemm ? (size_t)OC * parts : 0)) * slots * sizeof(float));
+            g.k_per_split = M;
+            g.sk_items = plan->d_items;
+            g.splits = slots;
+            {
+                llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
+                constexpr int SMEM = gemmk::smem_bytes(256, 256, 8);
+                if (dbias_in_gemm) {
+                    g.rowsum = g.partial + mn * slots;            // [slots * parts][OC]
+                    auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL_ROWSUM>;
+                    static bool attr_set = false;
+                    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
+                    kern<<<plan->G, 512, SMEM, st>>>(g);
+                } else {
+                    auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL>;
+                    static bool attr_set = false;
+                    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
+                    kern<<<plan->G, 512, SMEM, st>>>(g);
+                }
+                LAUNCH_CHECK();
+            }
+            llmk::ProfScope prof("splitk_reduce", 0, (double)mn * slots * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
+            const unsigned main_blocks = (unsigned)CEIL_DIV(mn / 4, (size_t)256);
+            const unsigned bias_blocks = dbias_in_gemm ? (unsigned)CEIL_DIV(OC, SKR_ROWS) : 0u;
+            splitk_reduce_kernel<true><<<main_blocks + bias_blocks, 256, 0, st>>>((floatX*)dweight, g.partial, mn, slots,
+                                                                               (floatX*)dbias, g.rowsum, OC, slots * parts, main_blocks);
+            LAUNCH_CHECK();
+#endif
         } else {
             const size_t mn = (size_t)OC * C;
             const int parts = big ? 4 : 2;                        // column waves of the tile configuration: each leaves a partial

@@ -57,7 +57,12 @@ struct GemmArgs {
     float* rowsum;        // [splits * WGN][M] fp32 (WGN: column waves of the tile configuration)  (EPI_PARTIAL_ROWSUM)
     int k_per_split;      // multiple of the K block
     int splits;
+    // A work list made by the host (EPI_PARTIAL*), or null: workgroup list c = xcd * (grid / 8) + index within the XCD takes
+    // the items sk_items[c][0..SK_MAX_ITEMS) in turn, two words each: tile row | tile column << 12 | partial slot << 24, and
+    // first K block | number of K blocks << 16 (a count of 0 ends the list). `splits` is the number of partial slots.
+    const unsigned* sk_items;
 };
+constexpr int SK_MAX_ITEMS = 8;
 
 #if !defined(LLMK_FP32)
 
@@ -170,7 +175,21 @@ gemm_pipelined_kernel(GemmArgs g) {
     // crosses HBM once. Otherwise XCD x takes the ids [x*G/8, (x+1)*G/8) of every round, so that a split's tiles
     // (which share their K range of both operands) sit on one XCD.
     const int G = gridDim.x;
-    auto work_item = [&](int it, int& tm, int& tn, int& sp) -> bool {
+    auto work_item = [&](int it, int& tm, int& tn, int& sp, int& kb, int& nk) -> bool {
+        if constexpr (IS_PARTIAL) {
+            if (g.sk_items) {                                     // the host's list: ranges of K of any length
+                if (it >= SK_MAX_ITEMS) return false;
+                const int c = (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3);
+                const unsigned* q = g.sk_items + ((size_t)c * SK_MAX_ITEMS + it) * 2;
+                const unsigned w0 = q[0], w1 = q[1];
+                nk = (int)(w1 >> 16);
+                if (nk == 0) return false;
+                tm = (int)(w0 & 0xfff); tn = (int)((w0 >> 12) & 0xfff); sp = (int)(w0 >> 24);
+                kb = (int)(w1 & 0xffff) * PBK;
+                return true;
+            }
+        }
+        auto k_range = [&](int split) { kb = split * g.k_per_split; nk = (min(g.K, kb + g.k_per_split) - kb) / PBK; };
         const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3, per_x = G >> 3;
         if (g.splits == 1 && tiles_m >= 64) {
             const int r0 = (tiles_m * xcd) >> 3, rows = ((tiles_m * (xcd + 1)) >> 3) - r0;
@@ -179,12 +198,14 @@ gemm_pipelined_kernel(GemmArgs g) {
             tile_of(q, rows, tiles_n, tm, tn);
             tm += r0;
             sp = 0;
+            k_range(0);
             return true;
         }
         const int w = it * G + xcd * per_x + local;
         if (w >= num_work) return false;
         tile_of(w % num_tiles, tiles_m, tiles_n, tm, tn);
         sp = w / num_tiles;
+        k_range(sp);
         return true;
     };
 
@@ -364,10 +385,8 @@ gemm_pipelined_kernel(GemmArgs g) {
     static_assert(CPW + NS_EPI <= 63, "vmcnt is a 6-bit counter");
 
     int it = 0;
-    int tile_m, tile_n, split;
-    if (!work_item(0, tile_m, tile_n, split)) return;
-    int kbeg = split * g.k_per_split;
-    int nkb = (min(g.K, kbeg + g.k_per_split) - kbeg) / PBK;
+    int tile_m, tile_n, split, kbeg, nkb;
+    if (!work_item(0, tile_m, tile_n, split, kbeg, nkb)) return;
     auto is_edge = [&](int tm, int tn) -> bool { return tm * BM + BM > g.M || tn * BN + BN > g.N; };
     bool voff_edge = is_edge(tile_m, tile_n);
     setup_bases(tile_m * BM, tile_n * BN, kbeg);
@@ -467,8 +486,8 @@ gemm_pipelined_kernel(GemmArgs g) {
         bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
         const int nst = nkb;
         // the next work item's coordinates are worked out here (integer divisions), under the K loop's MFMAs
-        int next_m, next_n, next_split;
-        const bool have_next = work_item(it + 1, next_m, next_n, next_split);
+        int next_m, next_n, next_split, next_kbeg = 0, next_nkb = 0;
+        const bool have_next = work_item(it + 1, next_m, next_n, next_split, next_kbeg, next_nkb);
         auto buf_idx = [&](int st) -> int { return (st + par) & 1; };
         auto buf_of = [&](int st) -> unsigned { return (unsigned)buf_idx(st) * STAGE; };
         // The last-but-one stage frees a buffer a whole stage before the tile ends: the next work item's first stage
@@ -477,11 +496,8 @@ gemm_pipelined_kernel(GemmArgs g) {
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
         constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
-        int next_kbeg = 0, next_nkb = 0;
         bool early0 = false;
         if (have_next) {
-            next_kbeg = next_split * g.k_per_split;
-            next_nkb = (min(g.K, next_kbeg + g.k_per_split) - next_kbeg) / PBK;
             if constexpr (EARLY0) {
                 early0 = nst >= 2 && !voff_edge && !is_edge(next_m, next_n);
                 if (early0) bases_into(tile_base_n, next_m * BM, next_n * BN, next_kbeg);

@@ -114,12 +114,23 @@ def test_forward_projection_with_gelu_epilogue(C, OC):
     G.check_no_error(L)
 
 
-@pytest.mark.parametrize("C,OC", LAYER_SHAPES)
-def test_backward_projection_is_the_integer_product(C, OC):
+@pytest.mark.parametrize("split_mode", [0, 1])
+@pytest.mark.parametrize("C,OC", LAYER_SHAPES + [(1600, 1600), (1600, 6400)])
+def test_backward_projection_is_the_integer_product(C, OC, split_mode):
     """dinp = dout . W (overwrites), dweight += dout^T . inp over 65536 rows (split K, partial sums in fp32), dbias +=
-    column sums of dout (taken inside the weight-gradient GEMM)."""
+    column sums of dout (taken inside the weight-gradient GEMM). Both ways of cutting the contraction into work items:
+    equal splits of every tile (0), one long and a few short pieces per tile where the shape allows them (1)."""
     import torch
     L = G.lib("bf16")
+    L.llmk_matmul_backward_split_mode(split_mode)
+    try:
+        _backward_projection_case(L, C, OC)
+    finally:
+        L.llmk_matmul_backward_split_mode(-1)
+
+
+def _backward_projection_case(L, C, OC):
+    import torch
     M = N_ROWS if C * OC <= 3072 * 768 else N_ROWS // 4
     x, w, g = ints((M, C), 7, -2, 2), ints((OC, C), 8), ints((M, OC), 9, -2, 2)
     dw0, db0 = ints((OC, C), 10, -50, 50), ints((OC,), 11, -50, 50)
