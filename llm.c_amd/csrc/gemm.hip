@@ -479,7 +479,7 @@ splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, 
 constexpr int SK_MIN_BLOCKS = 4;
 int g_sk_mode = -1;                  // llmk_matmul_backward_split_mode
 struct SkPlan {
-    int tiles_m = 0, tiles_n = 0, kblocks = 0, G = 0;
+    int tiles_m = 0, tiles_n = 0, kblocks = 0, G = 0, device = -1;
     int slots = 0;                   // pieces per tile
     double cost = 1e30;              // launch time in units of the perfectly balanced GEMM, partial passes included
     unsigned* d_items = nullptr;     // [G][SK_MAX_ITEMS][2]
@@ -526,9 +526,12 @@ void sk_build(SkPlan& p, int tiles_m, int tiles_n, int kblocks, int G, double pa
 // plans are kept for the life of the process (a training run has four to six shapes), their device copies with them
 SkPlan* sk_plan(int tiles_m, int tiles_n, int kblocks, int G, double pass) {
     static std::vector<SkPlan*> plans;
+    int device = 0;
+    (void)hipGetDevice(&device);                                  // the list lives in the memory of the GPU it was made on
     for (SkPlan* q : plans)
-        if (q->tiles_m == tiles_m && q->tiles_n == tiles_n && q->kblocks == kblocks && q->G == G) return q;
+        if (q->tiles_m == tiles_m && q->tiles_n == tiles_n && q->kblocks == kblocks && q->G == G && q->device == device) return q;
     SkPlan* p = new SkPlan();
+    p->device = device;
     sk_build(*p, tiles_m, tiles_n, kblocks, G, pass);
     plans.push_back(p);
     return p;
