@@ -74,6 +74,12 @@ __device__ __forceinline__ int fresh_lane(int lane) {
     asm volatile("" : "+v"(lane));
     return lane;
 }
+// max of a value with the one held by the lane 32 away (the other 16 keys of each 32-key block): one lane swap inside
+// the vector ALU instead of a trip through the LDS crossbar, which sits in every step's dependent chain
+__device__ __forceinline__ float fa_max_with_other_half(float v) {
+    const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+    return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+}
 // row index (within a 32-row block) of accumulator register r for this lane
 __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
 
@@ -341,7 +347,7 @@ fa_forward_kernel(floatX* __restrict__ out, float* __restrict__ stats, const flo
             float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
             for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
-            mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+            mx = fa_max_with_other_half(mx);
             const float m_top = fmaxf(m, mx * c);
             const bool outgrown = m_top > m + FA_MAX_SLACK;
             if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
@@ -496,7 +502,7 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
                 float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
                 for (int r = 1; r < 16; r++) mx = fmaxf(fmaxf(mx, sacc[0][r]), sacc[1][r]);     // v_max3_f32
-                mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
+                mx = fa_max_with_other_half(mx);
                 const float m_top = fmaxf(m, mx * c);
                 const bool outgrown = m_top > m + FA_MAX_SLACK;
                 if (__builtin_amdgcn_ballot_w64(outgrown) != 0) {   // some row's scores outgrew its reference point: rescale
