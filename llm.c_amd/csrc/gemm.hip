@@ -538,9 +538,12 @@ SkPlan* sk_plan(int tiles_m, int tiles_n, int kblocks, int G, double pass) {
 }
 bool sk_upload(SkPlan& p) {
     if (p.uploaded) return true;
-    if (hipMalloc(&p.d_items, p.items.size() * sizeof(unsigned)) != hipSuccess) return false;
+    // no room or no copy: the caller falls back to equal splits, and the error must not surface at its launch check
+    if (hipMalloc(&p.d_items, p.items.size() * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); p.valid = false; return false; }
     // a synchronous copy, once per shape
-    if (hipMemcpy(p.d_items, p.items.data(), p.items.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess) return false;
+    if (hipMemcpy(p.d_items, p.items.data(), p.items.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess) {
+        (void)hipGetLastError(); p.valid = false; return false;
+    }
     p.uploaded = true;
     return true;
 }
