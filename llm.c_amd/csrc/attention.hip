@@ -77,8 +77,12 @@ __device__ __forceinline__ int fresh_lane(int lane) {
 // max of a value with the one held by the lane 32 away (the other 16 keys of each 32-key block): one lane swap inside
 // the vector ALU instead of a trip through the LDS crossbar, which sits in every step's dependent chain
 __device__ __forceinline__ float fa_max_with_other_half(float v) {
-    const auto sw = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
-    return fmaxf(__builtin_bit_cast(float, sw[0]), __builtin_bit_cast(float, sw[1]));
+    // As an instruction, not through __builtin_amdgcn_permlane32_swap: this compiler hands back the first result for both
+    // elements of the builtin's pair, which silently drops the maximum (and overflows the exponentials as soon as scores
+    // are large). The two wait states are the ones the compiler puts between a vector write and this instruction.
+    unsigned a = __builtin_bit_cast(unsigned, v), b = a;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+    return fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b));
 }
 // row index (within a 32-row block) of accumulator register r for this lane
 __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }

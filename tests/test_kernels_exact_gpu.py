@@ -266,6 +266,31 @@ def test_attention_at_the_benchmark_shapes(B, T, NH):
     G.check_no_error(L)
 
 
+@pytest.mark.parametrize("T", [1024, 320])
+def test_attention_with_large_scores(T):
+    """Scores whose spread (hundreds of nats inside a row) is far beyond what an exponential survives without the row's
+    true running maximum: a reference point taken from only part of a key block, or one that lags, overflows here, where
+    ordinary-sized inputs would still give the right answer. Forward output against the fp32 formulation, every value
+    finite. T = 1024 takes the direct-to-LDS kernel, T = 320 the register-staged one."""
+    import torch
+    L = G.lib("bf16")
+    B, NH = 4, 6
+    Cc = NH * 64
+    gen = torch.Generator(device="cuda"); gen.manual_seed(T)
+    qkv = torch.randn((B, T, 3 * Cc), generator=gen, device="cuda")
+    qkv[:, :, :2 * Cc] *= 8.0                                  # q and k: scores of +-60 nats rms, several hundred at the extremes
+    qkv = qkv.to(torch.bfloat16)
+    out = torch.zeros((B, T, Cc), dtype=torch.bfloat16, device="cuda")
+    stats = torch.zeros((B, NH, T), dtype=torch.float32, device="cuda")
+    L.llmk_attention_forward(G.ptr(out), G.ptr(stats), G.ptr(qkv), B, T, NH, Cc, None)
+    G.sync()
+    assert torch.isfinite(out.float()).all() and torch.isfinite(stats).all()
+    r_out, r_lse, _ = torch_attention(qkv, torch.zeros((B, T, Cc), dtype=torch.bfloat16, device="cuda"), NH)
+    assert rel_fro(out, r_out) < 1e-2
+    assert ((stats - r_lse).abs() / r_lse.abs().clamp_min(1.0)).max().item() < 1e-2
+    G.check_no_error(L)
+
+
 @pytest.mark.parametrize("zero", ["Q", "K"])
 def test_attention_exact_zeros(zero):
     """Q = 0: all scores are 0, every row is the running mean of V, and dK = scale * dS^T Q is exactly zero;
