@@ -25,6 +25,10 @@
  *                             bit-equality of its fp32 state with the fp32 update (itself held to train_gpt2.c's
  *                             AdamW over several steps) and of its bf16 parameter with the stochastic rounding of
  *                             that state; the rounding by its exact up-probability low16/65536.
+ *   bf16 rounding,            cref_f32_to_bf16[_array]: an independent library cast on a million bit patterns, every
+ *   sum of squares            exact tie of eight exponents in both parities, infinities, denormals, NaNs;
+ *                             cref_sum_squares: numpy's float64 sum on inputs where a float accumulator differs in
+ *                             the 6th digit, and the closed form of 1^2 + ... + n^2 (same test file).
  */
 #include <math.h>
 #include <stdint.h>

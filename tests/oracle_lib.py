@@ -48,6 +48,8 @@ def cref():
     L = C.CDLL(CREF_SO)
     L.cref_f32_to_bf16_array.argtypes = [u16p, f32p, C.c_size_t]
     L.cref_bf16_to_f32_array.argtypes = [f32p, u16p, C.c_size_t]
+    L.cref_f32_to_bf16.argtypes = [C.c_float]
+    L.cref_f32_to_bf16.restype = C.c_uint16
     L.cref_mt_kat.argtypes = [C.c_uint32, u32p, f32p, u32p, f32p, u32p]
     L.cref_param_sizes.argtypes = [np.ctypeslib.ndpointer(dtype=np.uint64), C.POINTER(Config)]
     L.cref_param_sizes.restype = C.c_size_t

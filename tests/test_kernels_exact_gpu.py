@@ -266,19 +266,33 @@ def test_attention_at_the_benchmark_shapes(B, T, NH):
     G.check_no_error(L)
 
 
+@pytest.mark.parametrize("pattern", ["random", "rising", "falling"])
 @pytest.mark.parametrize("T", [1024, 320])
-def test_attention_with_large_scores(T):
+def test_attention_with_large_scores(T, pattern):
     """Scores whose spread (hundreds of nats inside a row) is far beyond what an exponential survives without the row's
     true running maximum: a reference point taken from only part of a key block, or one that lags, overflows here, where
-    ordinary-sized inputs would still give the right answer. Forward output against the fp32 formulation, every value
-    finite. T = 1024 takes the direct-to-LDS kernel, T = 320 the register-staged one."""
+    ordinary-sized inputs would still give the right answer. Forward output against the fp32 formulation
+    (train_gpt2.c:271-345), every value finite. T = 1024 takes the direct-to-LDS kernel, T = 320 the register-staged one.
+      random:  q and k scaled by 8, scores of +-60 nats rms.
+      rising:  every row's scores grow along the keys by about 0.3 nats per key (plus noise), 19 nats per 64-key step,
+               so every step of the key loop moves the reference point, by more than any slack it is allowed to lag.
+      falling: the mirror image, the first key dominates by up to 300 nats and the reference point never moves again;
+               every later probability underflows and the output is the first value row."""
     import torch
     L = G.lib("bf16")
     B, NH = 4, 6
     Cc = NH * 64
     gen = torch.Generator(device="cuda"); gen.manual_seed(T)
     qkv = torch.randn((B, T, 3 * Cc), generator=gen, device="cuda")
-    qkv[:, :, :2 * Cc] *= 8.0                                  # q and k: scores of +-60 nats rms, several hundred at the extremes
+    if pattern == "random":
+        qkv[:, :, :2 * Cc] *= 8.0                              # q and k: scores of +-60 nats rms, several hundred at the extremes
+    else:
+        # q = 8 u + noise, k_t = +-0.3 t u + noise with u a unit vector per head: score(q, k_t) = q.k_t / 8 = +-0.3 t + O(1)
+        u = torch.randn((NH, 64), generator=gen, device="cuda")
+        u = (u / u.norm(dim=1, keepdim=True)).view(1, 1, Cc)
+        t = torch.arange(T, device="cuda", dtype=torch.float32).view(1, T, 1)
+        qkv[:, :, :Cc] = 8.0 * u + 0.5 * qkv[:, :, :Cc]
+        qkv[:, :, Cc:2 * Cc] = (0.3 if pattern == "rising" else -0.3) * t * u + 0.5 * qkv[:, :, Cc:2 * Cc]
     qkv = qkv.to(torch.bfloat16)
     out = torch.zeros((B, T, Cc), dtype=torch.bfloat16, device="cuda")
     stats = torch.zeros((B, NH, T), dtype=torch.float32, device="cuda")
@@ -288,6 +302,9 @@ def test_attention_with_large_scores(T):
     r_out, r_lse, _ = torch_attention(qkv, torch.zeros((B, T, Cc), dtype=torch.bfloat16, device="cuda"), NH)
     assert rel_fro(out, r_out) < 1e-2
     assert ((stats - r_lse).abs() / r_lse.abs().clamp_min(1.0)).max().item() < 1e-2
+    if pattern != "random":
+        spread = (r_lse.max() - r_lse.min()).item()
+        assert spread > 60.0, spread                           # the rows' reference points do span the range claimed
     G.check_no_error(L)
 
 

@@ -410,8 +410,16 @@ def test_attention_forward_backward(precision, B, T, NH):
     close(got, rd, **tol(precision, 1e-4 * scale, bf16_rel=1.0 / 32, bf16_atol=2e-2 * scale), what="dqkv")
     for i, name in enumerate(("dQ", "dK", "dV")):          # per gradient, over the whole tensor: bf16 operands and probabilities
         a, r = got[..., i * Cc:(i + 1) * Cc], rd[..., i * Cc:(i + 1) * Cc]
-        # relative to the gradient's own norm, or to a twentieth of all three where it vanishes (T = 1: dQ = dK = 0)
-        e = float(np.linalg.norm((a - r).ravel()) / max(np.linalg.norm(r.ravel()), 0.05 * np.linalg.norm(rd.ravel())))
+        joint = np.linalg.norm(rd.ravel())
+        if np.linalg.norm(r.ravel()) < 1e-3 * joint:
+            # T = 1: one key, probability 1, so dS = P (dP - D) is mathematically 0 and so are dQ and dK. The kernels
+            # form dP - D from two fp32 sums of the same 64 products taken in different orders, which leaves a
+            # rounding residue (1e-7 of the joint norm measured in fp32) instead of an exact zero; the oracle's loop
+            # (train_gpt2.c:347-405) gives exact zeros. Held to: no more than fp32 / bf16 rounding of the joint norm.
+            e = float(np.linalg.norm((a - r).ravel()) / joint)
+            assert e < (1e-6 if precision == "fp32" else 2e-3), (name, "vanishing gradient", e)
+            continue
+        e = float(np.linalg.norm((a - r).ravel()) / np.linalg.norm(r.ravel()))
         assert e < (2e-5 if precision == "fp32" else 1e-2), (name, e)
     # causality at the kernel level: future tokens do not change earlier outputs
     if T >= 64:

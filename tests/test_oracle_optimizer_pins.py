@@ -13,6 +13,9 @@ here, so each function is fixed by something that does not restate its own formu
     low-precision parameter the stochastic rounding of that state with the element's noise word; the fp32 update
     itself is held to the plain AdamW of train_gpt2.c:1007-1033 (pinned against the compiled reference in
     test_oracle_vs_reference.py) over several steps with non-zero state, decay and gradient scale.
+  * the two helpers every optimiser check leans on: cref_f32_to_bf16[_array] (round to nearest even, quiet NaNs)
+    against an independent cast, ties and special values included; cref_sum_squares against a float64 sum and a
+    closed form.
 """
 import numpy as np
 
@@ -207,3 +210,74 @@ def test_adamw_mixed_is_the_f32_update_plus_stochastic_rounding():
             got = mp.astype(np.uint32)
             assert np.all((got == lo) | (got == lo + 1))
             assert 0.2 < np.mean(got == lo + 1) < 0.8                                    # both neighbours occur
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# cref_sum_squares and cref_f32_to_bf16[_array]: the two helpers the optimiser tests lean on
+# ---------------------------------------------------------------------------------------------------------------------
+def test_sum_squares_is_the_double_precision_sum():
+    """dev/cuda/global_norm.cu:21-28 accumulates in double. Checked against numpy's float64 sum, on inputs where a
+    float accumulator is visibly off: 300000 values of 1 + 2^-12 k/n summed in fp32 lose the 6th digit."""
+    L = ol.cref()
+    n = 300000
+    x = (1.0 + np.arange(n, dtype=np.float64) / n * 2.0 ** -12).astype(np.float32)
+    want = float(np.sum(x.astype(np.float64) ** 2))
+    got = L.cref_sum_squares(x, n)
+    assert abs(got - want) <= 1e-12 * want
+    naive = float(np.cumsum((x * x).astype(np.float32), dtype=np.float32)[-1])
+    assert abs(naive - want) > 1e-6 * want                              # the case separates float from double
+    # signs, magnitudes 1e-20 ... 1e+18 and a closed form: sum of k^2 for k = 1..n is n(n+1)(2n+1)/6
+    r = np.random.default_rng(5)
+    y = (r.standard_normal(100003) * 10.0 ** r.uniform(-20, 18, 100003)).astype(np.float32)
+    want = float(np.sum(y.astype(np.float64) ** 2))
+    assert abs(L.cref_sum_squares(y, y.size) - want) <= 1e-12 * want
+    k = np.arange(1, 2001, dtype=np.float32)
+    assert L.cref_sum_squares(k, k.size) == 2000 * 2001 * 4001 / 6
+    assert L.cref_sum_squares(k, 0) == 0.0
+
+
+def test_f32_to_bf16_rounds_to_nearest_even_like_the_library_cast():
+    """__float2bfloat16_rn (what the reference's (floatX) casts compile to, llmc/cuda_common.h:82-92) is IEEE
+    round-to-nearest-even with quiet NaNs. Checked against torch's cast (an independent implementation) on random bit
+    patterns and on the cases a rounding mistake shows in: every exact tie of several exponents with both parities of
+    the kept bit, the values one unit either side of a tie, +-0, +-inf, denormals, the carry into the exponent and
+    into infinity, NaNs."""
+    import torch
+    L = ol.cref()
+    r = np.random.default_rng(11)
+    bits = [r.integers(0, 2 ** 32, 1 << 20, dtype=np.uint64).astype(np.uint32)]
+    for e in (0, 1, 37, 126, 127, 128, 200, 254):                       # exponent fields incl. denormal and the largest
+        for sign in (0, 1):
+            hi = (np.arange(128, dtype=np.uint32) | np.uint32(e << 7) | np.uint32(sign << 15)) << 16  # all 7-bit mantissas
+            for low in (0x0000, 0x0001, 0x7fff, 0x8000, 0x8001, 0xffff):
+                bits.append(hi | np.uint32(low))
+    bits.append(np.array([0x00000000, 0x80000000, 0x7f800000, 0xff800000, 0x00000001, 0x80000001, 0x007fffff,
+                          0x7f7fffff, 0xff7fffff, 0x7f7f8000, 0x7f7f7fff, 0x3f7fffff, 0x3f7f8000], np.uint32))
+    bits = np.concatenate(bits)
+    x = bits.view(np.float32)
+    got = np.zeros(x.size, np.uint16)
+    L.cref_f32_to_bf16_array(got, x, x.size)
+    want = torch.from_numpy(x.copy()).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    nan = (bits & 0x7fffffff) > 0x7f800000          # a NaN's payload is the implementation's choice: both must be NaN
+    assert nan.sum() > 1000 and np.array_equal(got[~nan], want[~nan])
+    assert np.all((got[nan] & 0x7f80) == 0x7f80) and np.all((got[nan] & 0x7f) != 0)
+    assert np.all((want[nan] & 0x7f80) == 0x7f80) and np.all((want[nan] & 0x7f) != 0)
+    # ties by hand: 1 + 2^-8 lies midway between 1 (kept bit 0) and 1 + 2^-7 -> down; 1 + 3*2^-8 -> up to 1 + 2^-6
+    assert L.cref_f32_to_bf16(np.float32(1 + 2.0 ** -8)) == 0x3f80
+    assert L.cref_f32_to_bf16(np.float32(1 + 3 * 2.0 ** -8)) == 0x3f82
+    assert L.cref_f32_to_bf16(np.float32(3.3895313892515355e38)) == 0x7f7f                 # largest bf16, exact
+    assert L.cref_f32_to_bf16(np.float32(3.4028234663852886e38)) == 0x7f80                 # FLT_MAX rounds to inf
+    # NaNs stay NaNs (quiet), whatever their payload, and keep their sign
+    nan_bits = np.array([0x7fc00000, 0x7f800001, 0x7f80ffff, 0xffc00000, 0xff800001, 0x7fffffff, 0x7fa00000], np.uint32)
+    out = np.zeros(nan_bits.size, np.uint16)
+    L.cref_f32_to_bf16_array(out, nan_bits.view(np.float32), nan_bits.size)
+    assert np.all((out & 0x7f80) == 0x7f80) and np.all((out & 0x007f) != 0)
+    assert np.array_equal(out >> 15, (nan_bits >> 31).astype(np.uint16))
+    # scalar and array forms agree, and widening is the inverse on representable values
+    for i in range(0, x.size, 9973):
+        assert L.cref_f32_to_bf16(x[i]) == got[i]
+    h = r.integers(0, 2 ** 16, 4096, dtype=np.uint32).astype(np.uint16)
+    h = h[(h & 0x7f80) != 0x7f80]
+    wide = np.zeros(h.size, np.float32); L.cref_bf16_to_f32_array(wide, h, h.size)
+    back = np.zeros(h.size, np.uint16); L.cref_f32_to_bf16_array(back, wide, h.size)
+    assert np.array_equal(back, h) and np.array_equal(wide.view(np.uint32), h.astype(np.uint32) << 16)
