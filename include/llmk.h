@@ -15,10 +15,15 @@
  *   - the caller owns every buffer; functions enqueue work on `stream` and return without
  *     waiting (exception: llmk_encoder_backward builds its buckets on the host first);
  *   - a single host thread drives the library;
- *   - no entry point here allocates device memory per call. GEMMs whose output is smaller than
- *     the machine (weight gradients) split the contraction and use one library-owned
- *     workspace that grows to the largest request seen and is then reused (the role of the
- *     reference's cublaslt_workspace, llmc/cublas_common.h:28-31);
+ *   - no entry point here allocates device memory per call. Two launchers take scratch from ONE
+ *     library-owned workspace (the role of the reference's cublaslt_workspace,
+ *     llmc/cublas_common.h:28-31): llmk_matmul_backward (fp32 partial products of the split
+ *     weight gradient) and llmk_attention_backward (one float per query and head). The
+ *     workspace grows to the largest request seen (a free, an allocation and a device
+ *     synchronisation at that call) and is then reused; a caller that must not allocate inside
+ *     a step sizes it beforehand with llmk_workspace_reserve() from the
+ *     llmk_*_workspace_bytes() of its shapes, as gpt2_allocate_state does. Nothing else is
+ *     allocated or copied behind the caller's back: work lists are derived in the kernels;
  *   - errors: a failed HIP call or a violated shape precondition prints a message and exits
  *     (llmc/cuda_common.h:52-58). llmk_set_error_mode(1) makes the library record the
  *     message and return instead, for tests; read it with llmk_last_error().
@@ -42,6 +47,10 @@ extern "C" {
 /* Selects the device and reads its properties (reference: common_start, train_gpt2.cu:1173-1200). */
 void llmk_init(int device);
 void llmk_shutdown(void);
+/* The library workspace (see the contract above): grow it to at least `bytes` now / its present size. The reference
+ * allocates its cuBLASLt workspace once at start-up (llmc/cublas_common.h:28-31, train_gpt2.cu:1190-1195). */
+void llmk_workspace_reserve(size_t bytes);
+size_t llmk_workspace_bytes(void);
 /* "bf16" or "fp32": the floatX of this shared object (reference: PRECISION_MODE, llmc/cuda_common.h:68-92) */
 const char* llmk_precision(void);
 /* sizeof(floatX) */
@@ -140,6 +149,11 @@ size_t llmk_matmul_backward_bias_scratch_floats(int OC);
  * them. The result is the same sum in a different (fixed) order of fp32 partials. No counterpart in the reference
  * (cuBLASLt chooses its own split there); for tests and tuning. */
 void llmk_matmul_backward_split_mode(int mode);
+/* What the last llmk_matmul_backward did with the weight gradient's contraction: *kind = 0 not cut, 1 equal splits,
+ * 2 one long and several short pieces per tile; *pieces = fp32 partials per output element. For tests. */
+void llmk_matmul_backward_last_split(int* kind, int* pieces);
+/* Upper bound of the workspace llmk_matmul_backward(B, T, C, OC) asks for, whichever way it cuts K. */
+size_t llmk_matmul_backward_workspace_bytes(int B, int T, int C, int OC);
 
 /* gelu_backward_inplace (llmc/gelu.cuh:59) and the bias gradient of matmul_backward (llmc/matmul.cuh:251-266) in
  * one pass over (B*T, OC): d_in_out *= gelu'(inp), then dbias[OC] += column sums of the result. Same values as
@@ -161,6 +175,7 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
  * Uses B*NH*T floats of the library workspace for the rowsum(dO*O) term. */
 void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                              int B, int T, int NH, int C, void* stream);
+size_t llmk_attention_backward_workspace_bytes(int B, int T, int NH);
 
 /* attention_forward, llmc/attention.cuh:195: the launcher of reference builds without cuDNN, same argument order.
  * inp (B,T,3C) Q, K, V as the qkv projection wrote them; out (B,T,C). qkvr (B*T*3C elements) and att (B*NH*T*T elements)

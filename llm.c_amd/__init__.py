@@ -42,6 +42,11 @@ KERNEL_ABI = {
     "llmk_clear_error": (None, []),
     "llmk_profile_enable": (None, [i32]),
     "llmk_matmul_backward_split_mode": (None, [i32]),
+    "llmk_matmul_backward_last_split": (None, [ip, ip]),
+    "llmk_matmul_backward_workspace_bytes": (sz, [i32, i32, i32, i32]),
+    "llmk_attention_backward_workspace_bytes": (sz, [i32, i32, i32]),
+    "llmk_workspace_reserve": (None, [sz]),
+    "llmk_workspace_bytes": (sz, []),
     "llmk_profile_only": (None, [C.c_char_p]),
     "llmk_zero": (None, [vp, C.c_size_t, vp]),
     "llmk_probe_mfma_peak": (None, [C.POINTER(C.c_double), vp, vp]),

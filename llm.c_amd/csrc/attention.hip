@@ -1384,6 +1384,10 @@ void llmk_attention_forward(void* out, float* stats, const void* inp, int B, int
     LAUNCH_CHECK();
 }
 
+size_t llmk_attention_backward_workspace_bytes(int B, int T, int NH) {
+    return (size_t)B * NH * T * sizeof(float);                   // rowsum(dO * O), one float per (batch, head, query)
+}
+
 void llmk_attention_backward(void* dqkvr, const void* dout, const void* qkvr, const void* o, const float* stats,
                              int B, int T, int NH, int C, void* stream) {
     attention_backward_impl(dqkvr, dout, qkvr, o, stats, B, T, NH, C, stream, nullptr);

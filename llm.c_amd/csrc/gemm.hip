@@ -479,75 +479,53 @@ splitk_reduce_kernel(floatX* __restrict__ C, const float* __restrict__ partial, 
 constexpr int SK_MIN_BLOCKS = 4;
 int g_sk_mode = -1;                  // llmk_matmul_backward_split_mode
 struct SkPlan {
-    int tiles_m = 0, tiles_n = 0, kblocks = 0, G = 0, device = -1;
     int slots = 0;                   // pieces per tile
+    int long_blocks = 0;             // K blocks of the long piece
+    int each = 0;                    // short pieces per workgroup
     double cost = 1e30;              // launch time in units of the perfectly balanced GEMM, partial passes included
-    unsigned* d_items = nullptr;     // [G][SK_MAX_ITEMS][2]
-    std::vector<unsigned> items;
-    bool valid = false, uploaded = false;
+    bool valid = false;
 };
-void sk_build(SkPlan& p, int tiles_m, int tiles_n, int kblocks, int G, double pass) {
-    p.tiles_m = tiles_m; p.tiles_n = tiles_n; p.kblocks = kblocks; p.G = G; p.valid = false;
+// Pure arithmetic on the shape: nothing is allocated or copied, the kernel derives each workgroup's pieces from
+// (tiles, long_blocks, each, slots) by the same enumeration (gemm_pipelined.hpp, work_item).
+SkPlan sk_build(int tiles_m, int tiles_n, int kblocks, int G, double pass) {
+    SkPlan p;
     const int T = tiles_m * tiles_n, S = kblocks;
-    if (tiles_m >= 4096 || tiles_n >= 4096 || S >= 65536 || T >= G || T * 8 < G) return;
-    int best_s = 0, best_x = 0, best_p = 0;
+    if (T >= G || T * 8 < G) return p;
     for (int s = 2; s <= 6; s++) {
         const int ny = T * (s - 1), p_each = CEIL_DIV(ny, G - T);
-        if (p_each + 1 > SK_MAX_ITEMS) continue;
+        if (p_each > SK_MAX_ITEMS) continue;
         int x = (int)((long long)p_each * S / (s - 1 + p_each));           // long piece = p short ones
         const int y_max = CEIL_DIV(S - x, s - 1), y_min = (S - x) / (s - 1);
         if (x < SK_MIN_BLOCKS || y_min < SK_MIN_BLOCKS) continue;
         const int makespan = std::max(x, p_each * y_max);
         const double cost = (double)makespan * G / ((double)T * S) + pass * s;
-        if (cost < p.cost) { p.cost = cost; best_s = s; best_x = x; best_p = p_each; }
+        if (cost < p.cost) { p.cost = cost; p.slots = s; p.long_blocks = x; p.each = p_each; p.valid = true; }
     }
-    if (!best_s) return;
-    const int s = best_s, x = best_x;
-    p.slots = s;
-    p.items.assign((size_t)G * SK_MAX_ITEMS * 2, 0u);
-    auto put = [&](int c, int n, int t, int slot, int k0, int len) {
-        const unsigned tm = (unsigned)(t / tiles_n), tn = (unsigned)(t % tiles_n);
-        p.items[((size_t)c * SK_MAX_ITEMS + n) * 2] = tm | (tn << 12) | ((unsigned)slot << 24);
-        p.items[((size_t)c * SK_MAX_ITEMS + n) * 2 + 1] = (unsigned)k0 | ((unsigned)len << 16);
-    };
-    for (int t = 0; t < T; t++) put(t, 0, t, 0, 0, x);                      // list t: the long piece of tile t
-    // the short pieces in (K range, tile) order, best_p at a time to the remaining lists
-    int c = T, n = 0;
-    for (int j = 1; j < s; j++) {
-        const int k0 = x + (int)((long long)(S - x) * (j - 1) / (s - 1)), k1 = x + (int)((long long)(S - x) * j / (s - 1));
-        for (int t = 0; t < T; t++) {
-            if (n == best_p) { c++; n = 0; }
-            if (c >= G) return;                                            // cannot happen: (G - T) * best_p >= T * (s - 1)
-            put(c, n++, t, j, k0, k1 - k0);
-        }
-    }
-    p.valid = true;
-}
-// plans are kept for the life of the process (a training run has four to six shapes), their device copies with them
-SkPlan* sk_plan(int tiles_m, int tiles_n, int kblocks, int G, double pass) {
-    static std::vector<SkPlan*> plans;
-    int device = 0;
-    (void)hipGetDevice(&device);                                  // the list lives in the memory of the GPU it was made on
-    for (SkPlan* q : plans)
-        if (q->tiles_m == tiles_m && q->tiles_n == tiles_n && q->kblocks == kblocks && q->G == G && q->device == device) return q;
-    SkPlan* p = new SkPlan();
-    p->device = device;
-    sk_build(*p, tiles_m, tiles_n, kblocks, G, pass);
-    plans.push_back(p);
     return p;
 }
-bool sk_upload(SkPlan& p) {
-    if (p.uploaded) return true;
-    // no room or no copy: the caller falls back to equal splits, and the error must not surface at its launch check
-    if (hipMalloc(&p.d_items, p.items.size() * sizeof(unsigned)) != hipSuccess) { (void)hipGetLastError(); p.valid = false; return false; }
-    // a synchronous copy, once per shape
-    if (hipMemcpy(p.d_items, p.items.data(), p.items.size() * sizeof(unsigned), hipMemcpyHostToDevice) != hipSuccess) {
-        (void)hipGetLastError(); p.valid = false; return false;
-    }
-    p.uploaded = true;
-    return true;
-}
 #endif
+
+// Equal splits of the weight gradient's K = B*T so that the work items fill whole rounds of the persistent launch (27
+// tiles -> 9 splits = 243 items on 256 CUs; 591 tiles -> 3 splits, 1773 items = 6.9 rounds instead of 3 rounds at 77 %;
+// 175 tiles -> 4 splits). Each split costs one fp32 pass over the output (8 bytes per element written and read back,
+// against 2*M flop per element in the GEMM): 800/M of the GEMM's time at the rates measured, 1.2 % at M = 65536.
+int tn_equal_splits(int M, size_t tiles, int num_cu, double* cost_out) {
+    int splits = 1;
+    double best = 1e30;
+    const double pass = 800.0 / (double)M;
+    for (int s = 1; s <= 32; s++) {
+        const size_t work = tiles * s, rounds = CEIL_DIV(work, (size_t)num_cu);
+        const double cost = (double)(rounds * num_cu) / (double)work + pass * s;
+        if (cost < best) { best = cost; splits = s; }
+    }
+    if (cost_out) *cost_out = best;
+    const int ksteps = CEIL_DIV(M, K_STEP);
+    splits = min(splits, max(1, ksteps / 8));                     // at least 8 K steps per split
+    return CEIL_DIV(ksteps, CEIL_DIV(ksteps, splits));
+}
+
+// what the last weight-gradient GEMM did with K: 0 = not cut, 1 = equal splits, 2 = one long + short pieces
+int g_last_split_kind = 0, g_last_split_pieces = 0;
 
 // ---- bias gradient: column sums of dout[N][OC] -----------------------------------------------
 // HBM-bound streaming reduction. Workgroup = 32 column-vectors (512 B of a row) x 8 row lanes; each lane keeps
@@ -759,6 +737,26 @@ void llmk_matmul_backward_split_mode(int mode) {
 #endif
 }
 
+void llmk_matmul_backward_last_split(int* kind, int* pieces) {
+    if (kind) *kind = g_last_split_kind;
+    if (pieces) *pieces = g_last_split_pieces;
+}
+
+size_t llmk_matmul_backward_workspace_bytes(int B, int T, int C, int OC) {
+    const int M = B * T, num_cu = llmk::device_info().num_cu;
+    if (M <= 0 || C <= 0 || OC <= 0) return 0;
+    const size_t tiles_big = (size_t)CEIL_DIV(OC, BIG_TILE) * CEIL_DIV(C, BIG_TILE);
+    const size_t tiles_small = (size_t)CEIL_DIV(OC, SMALL_TILE) * CEIL_DIV(C, SMALL_TILE);
+    int pieces = tn_equal_splits(M, tiles_big >= 8 ? tiles_big : tiles_small, num_cu, nullptr);
+#if !defined(LLMK_FP32)
+    if (tiles_big >= 8 && M % K_STEP == 0) {
+        const SkPlan plan = sk_build(CEIL_DIV(OC, BIG_TILE), CEIL_DIV(C, BIG_TILE), M / K_STEP, num_cu & ~7, 800.0 / (double)M);
+        if (plan.valid) pieces = max(pieces, plan.slots);
+    }
+#endif
+    return ((size_t)OC * C + (size_t)OC * 4) * pieces * sizeof(float);     // partial products + the bias gradient's row sums
+}
+
 void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
                           const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
                           const void* pre_gelu, int gelu_fusion) {
@@ -835,47 +833,28 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         const size_t tiles_small = (size_t)CEIL_DIV(OC, SMALL_TILE) * CEIL_DIV(C, SMALL_TILE);
         const bool big = tiles_big >= 8;                          // split-K fills the machine when there are few big tiles
         const size_t tiles = big ? tiles_big : tiles_small;
-        // Split K so that the work items fill whole rounds of the persistent launch (27 tiles -> 9 splits = 243 items on
-        // 256 CUs; 591 tiles -> 3 splits, 1773 items = 6.9 rounds instead of 3 rounds at 77 %; 175 tiles -> 4 splits).
-        // Each split costs one fp32 pass over the output (8 bytes per element written and read back, against 2*M flop
-        // per element in the GEMM): 800/M of the GEMM's time at the rates measured, 1.2 % at M = 65536.
-        int splits = 1;
-        {
-            double best = 1e30;
-            const double pass = 800.0 / (double)M;
-            for (int s = 1; s <= 32; s++) {
-                const size_t work = tiles * s, rounds = CEIL_DIV(work, (size_t)num_cu);
-                const double cost = (double)(rounds * num_cu) / (double)work + pass * s;
-                if (cost < best) { best = cost; splits = s; }
-            }
-        }
         double best_uniform = 1e30;
-        {
-            const size_t work = tiles * splits, rounds = CEIL_DIV(work, (size_t)num_cu);
-            best_uniform = (double)(rounds * num_cu) / (double)work + 800.0 / (double)M * splits;
-        }
-        const int ksteps = CEIL_DIV(M, K_STEP);
-        splits = min(splits, max(1, ksteps / 8));                 // at least 8 K steps per split
-        const int steps_per = CEIL_DIV(ksteps, splits);
-        splits = CEIL_DIV(ksteps, steps_per);
-        g.k_per_split = steps_per * K_STEP;
+        const int splits = tn_equal_splits(M, tiles, num_cu, &best_uniform);
+        g.k_per_split = CEIL_DIV(CEIL_DIV(M, K_STEP), splits) * K_STEP;
         const double tn_bytes = ((double)M * OC + (double)M * C + 2.0 * OC * C) * sizeof(floatX);
         if (splits == 1 && !tn_partial_always(g)) {
             LLMK_REQUIRE(!dbias_in_gemm, "matmul_backward: bias gradient was left to a kernel that is not being run");
             llmk::ProfScope prof("gemm_tn", 2.0 * M * (double)OC * C, tn_bytes, st);
             launch_best<true, true, EPI_ACCUM>(g, 1, big, st);
+            g_last_split_kind = 0; g_last_split_pieces = 1;
 #if !defined(LLMK_FP32)
-        } else if (SkPlan* plan = (big && M % K_STEP == 0 && pipelined_ok(g) && (!dbias || dbias_in_gemm) && g_sk_mode != 0)
-                                      ? sk_plan(CEIL_DIV(OC, BIG_TILE), CEIL_DIV(C, BIG_TILE), M / K_STEP, num_cu & ~7, 800.0 / (double)M)
-                                      : nullptr;
-                   plan && plan->valid && (g_sk_mode == 1 || plan->cost < 0.98 * best_uniform) && sk_upload(*plan)) {
-            // one long and s - 1 short pieces per tile, scheduled by the host's list (see sk_build)
+        } else if (const SkPlan plan = (big && M % K_STEP == 0 && pipelined_ok(g) && (!dbias || dbias_in_gemm) && g_sk_mode != 0)
+                                           ? sk_build(CEIL_DIV(OC, BIG_TILE), CEIL_DIV(C, BIG_TILE), M / K_STEP, num_cu & ~7, 800.0 / (double)M)
+                                           : SkPlan();
+                   plan.valid && (g_sk_mode == 1 || plan.cost < 0.98 * best_uniform)) {
+            // one long and s - 1 short pieces per tile (see sk_build)
             const size_t mn = (size_t)OC * C;
-            const int parts = 4, slots = plan->slots;
+            const int parts = 4, slots = plan.slots, G = num_cu & ~7;
             g.partial = (float*)llmk::workspace((mn + (dbias_in_gemm ? (size_t)OC * parts : 0)) * slots * sizeof(float));
             g.k_per_split = M;
-            g.sk_items = plan->d_items;
+            g.sk_tiles = CEIL_DIV(OC, BIG_TILE) * CEIL_DIV(C, BIG_TILE); g.sk_long = plan.long_blocks; g.sk_each = plan.each;
             g.splits = slots;
+            g_last_split_kind = 2; g_last_split_pieces = slots;
             {
                 llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
                 constexpr int SMEM = gemmk::smem_bytes(256, 256, 8);
@@ -884,12 +863,12 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
                     auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL_ROWSUM>;
                     static bool attr_set = false;
                     if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
-                    kern<<<plan->G, 512, SMEM, st>>>(g);
+                    kern<<<G, 512, SMEM, st>>>(g);
                 } else {
                     auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL>;
                     static bool attr_set = false;
                     if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
-                    kern<<<plan->G, 512, SMEM, st>>>(g);
+                    kern<<<G, 512, SMEM, st>>>(g);
                 }
                 LAUNCH_CHECK();
             }
@@ -903,6 +882,7 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         } else {
             const size_t mn = (size_t)OC * C;
             const int parts = big ? 4 : 2;                        // column waves of the tile configuration: each leaves a partial
+            g_last_split_kind = 1; g_last_split_pieces = splits;
             g.partial = (float*)llmk::workspace((mn + (dbias_in_gemm ? (size_t)OC * parts : 0)) * splits * sizeof(float));
             {
                 llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);

@@ -57,12 +57,13 @@ struct GemmArgs {
     float* rowsum;        // [splits * WGN][M] fp32 (WGN: column waves of the tile configuration)  (EPI_PARTIAL_ROWSUM)
     int k_per_split;      // multiple of the K block
     int splits;
-    // A work list made by the host (EPI_PARTIAL*), or null: workgroup list c = xcd * (grid / 8) + index within the XCD takes
-    // the items sk_items[c][0..SK_MAX_ITEMS) in turn, two words each: tile row | tile column << 12 | partial slot << 24, and
-    // first K block | number of K blocks << 16 (a count of 0 ends the list). `splits` is the number of partial slots.
-    const unsigned* sk_items;
+    // Uneven cut of K (EPI_PARTIAL*), or sk_tiles = 0: every one of the sk_tiles output tiles is cut at the same K blocks
+    // into one long piece of sk_long blocks (partial slot 0) and splits - 1 short ones that share the rest evenly (slot =
+    // rank along K). Workgroup list c = xcd * (grid / 8) + index within the XCD takes the long piece of tile c when
+    // c < sk_tiles; the others take sk_each consecutive short pieces, numbered (slot - 1) * sk_tiles + tile.
+    int sk_tiles, sk_long, sk_each;
 };
-constexpr int SK_MAX_ITEMS = 8;
+constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 
 #if !defined(LLMK_FP32)
 
@@ -177,15 +178,23 @@ gemm_pipelined_kernel(GemmArgs g) {
     const int G = gridDim.x;
     auto work_item = [&](int it, int& tm, int& tn, int& sp, int& kb, int& nk) -> bool {
         if constexpr (IS_PARTIAL) {
-            if (g.sk_items) {                                     // the host's list: ranges of K of any length
-                if (it >= SK_MAX_ITEMS) return false;
+            if (g.sk_tiles) {                                     // uneven cut: see GemmArgs
                 const int c = (int)(blockIdx.x & 7) * (G >> 3) + (int)(blockIdx.x >> 3);
-                const unsigned* q = g.sk_items + ((size_t)c * SK_MAX_ITEMS + it) * 2;
-                const unsigned w0 = q[0], w1 = q[1];
-                nk = (int)(w1 >> 16);
-                if (nk == 0) return false;
-                tm = (int)(w0 & 0xfff); tn = (int)((w0 >> 12) & 0xfff); sp = (int)(w0 >> 24);
-                kb = (int)(w1 & 0xffff) * PBK;
+                const int S = g.K / PBK;
+                int t;
+                if (c < g.sk_tiles) {
+                    if (it > 0) return false;
+                    t = c; sp = 0; kb = 0; nk = g.sk_long;
+                } else {
+                    const int q = (c - g.sk_tiles) * g.sk_each + it;
+                    if (it >= g.sk_each || q >= g.sk_tiles * (g.splits - 1)) return false;
+                    const int j = q / g.sk_tiles, rest = S - g.sk_long;
+                    t = q - j * g.sk_tiles; sp = j + 1;
+                    const int k0 = g.sk_long + (int)((long long)rest * j / (g.splits - 1));
+                    const int k1 = g.sk_long + (int)((long long)rest * (j + 1) / (g.splits - 1));
+                    kb = k0 * PBK; nk = k1 - k0;
+                }
+                tm = t / tiles_n; tn = t - tm * tiles_n;
                 return true;
             }
         }

@@ -146,6 +146,12 @@ void llmk_shutdown(void) {
     if (llmk::g_ws) { (void)hipFree(llmk::g_ws); llmk::g_ws = nullptr; llmk::g_ws_bytes = 0; }
 }
 
+void llmk_workspace_reserve(size_t bytes) {
+    if (llmk::failed()) return;
+    (void)llmk::workspace(bytes);
+}
+size_t llmk_workspace_bytes(void) { return llmk::g_ws_bytes; }
+
 const char* llmk_precision(void) { return LLMK_PRECISION_NAME; }
 int llmk_sizeof_floatx(void) { return (int)sizeof(floatX); }
 

@@ -407,6 +407,13 @@ void gpt2_allocate_state(LLMK_GPT2* m, int B, int T) {
     hipCheck(hipMalloc((void**)&m->m_memory, m->num_parameters * sizeof(float)));
     hipCheck(hipMalloc((void**)&m->v_memory, m->num_parameters * sizeof(float)));
     if (m->use_master_weights == 1) hipCheck(hipMalloc((void**)&m->master_weights, m->num_parameters * sizeof(float)));
+    // the library's workspace at its final size now, so that no training step allocates (the reference sizes its
+    // cuBLASLt workspace once, llmc/cublas_common.h:28-31)
+    const int C = m->config.channels, Vp = m->config.padded_vocab_size, NH = m->config.num_heads;
+    size_t ws = llmk_attention_backward_workspace_bytes(B, T, NH);
+    const int shapes[5][2] = {{C, 3 * C}, {C, C}, {C, 4 * C}, {4 * C, C}, {C, Vp}};
+    for (const auto& sh : shapes) ws = std::max(ws, llmk_matmul_backward_workspace_bytes(B, T, sh[0], sh[1]));
+    llmk_workspace_reserve(ws);
 }
 
 void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T) {
