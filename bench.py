@@ -3,7 +3,7 @@
 with the reference's CPU trainer timed beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-kernel-events] [--no-mfma-probe]
-                    [--no-other-configs] [--model d12|d24|d48 --batch B --recompute R]
+                    [--no-other-configs] [--no-microbench] [--model d12|d24|d48 --batch B --recompute R]
 
 A step = gpt2_forward + gpt2_backward_and_reduce + gpt2_calculate_grad_norm (clip at 1.0) + gpt2_update
 on one batch of synthetic tokens, exactly the work of one iteration of the reference's training loop
@@ -280,6 +280,9 @@ def main():
     ap.add_argument("--no-mfma-probe", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true",
                     help="skip the few steps of GPT-2 350M (B=32) and 1558M (B=16) that follow the headline measurement")
+    ap.add_argument("--no-microbench", action="store_true",
+                    help="skip the per-kernel table at the 124M shapes (BASELINE configs[1]) that follows the headline measurement")
+    ap.add_argument("--microbench-reps", type=int, default=5)
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first launch one copy kernel of known size (128 MiB read, 256 MiB written): the yardstick for "
                          "scaling FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run of this command")
@@ -349,6 +352,17 @@ def main():
             r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 2, False, lr=lr)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
                                                               "loss_first", "loss_last", "losses")})
+    if default_headline(args) and not args.no_microbench:
+        # BASELINE configs[1]: every launcher by itself at the 124M shapes, caches flushed before each repetition
+        # (llm.c_amd/microbench.py; the reference's dev/cuda/common.h:350-385 harness), after and outside the headline measurement
+        spec = importlib.util.spec_from_file_location("llmc_amd_microbench", os.path.join(ROOT, "llm.c_amd", "microbench.py"))
+        mb = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mb)
+        out["config1_microbench"] = [
+            {"case": r["case"], "family": r["kernel"], "launches": r["launches"], "median_ms": round(r["median_ms"], 5),
+             "min_ms": round(r["min_ms"], 5), "rate": round(r["rate"], 1), "unit": r["unit"], "bound": r["bound"],
+             "frac": round(r["frac"], 4)}
+            for r in mb.run_cases(L, reps=args.microbench_reps, emit=lambda line: print(line, file=sys.stderr, flush=True))]
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     C.CDLL(None).fflush(None)

@@ -821,13 +821,14 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
 #pragma unroll
                     for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
                 }
-                if (q0 < kw0 + 31 || q0 + 31 >= T) {            // diagonal block or rows past the end (wave-uniform test)
-                    const int ln = fresh_lane(lane), my_k = kw0 + (ln & 31);
+                if (q0 < kw0 + 31) {                             // diagonal block (wave-uniform test; T % 64 == 0: no rows past the end)
+                    asm volatile("" ::: "memory");                // keep this a branch: off the diagonal the selects are pure overhead
+                    // query q0 + acc_row(r) against key kw0 + idx: the lane's share of both sides is one small number
+                    const int ln = fresh_lane(lane);
+                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = kw0 - q0;
 #pragma unroll
-                    for (int r = 0; r < 16; r++) {
-                        const int q = q0 + acc_row(r, ln);
-                        if (q < my_k || q >= T) sacc[r] = 0.f;
-                    }
+                    for (int r = 0; r < 16; r++)
+                        if ((r >> 2) * 8 + (r & 3) + dl < lim) sacc[r] = 0.f;
                 }
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
@@ -1063,6 +1064,7 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
                 if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
+                    asm volatile("" ::: "memory");                // keep this a branch: off the diagonal the selects are pure overhead
                     const int ln = fresh_lane(lane);
                     const int dl = ((ln >> 5) << 2) - (ln & 31), lim = qw0 - k0;      // key k0 + acc_row(r) against query qw0 + idx
 #pragma unroll

@@ -34,16 +34,10 @@ PEAK_TFLOPS, PEAK_GBS = 2500.0, 8000.0
 MFMA_FAMILIES = ("gemm", "attention_forward", "attention_backward_dq", "attention_backward_dkdv")
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--reps", type=int, default=20)
-    ap.add_argument("--only", default="")
-    ap.add_argument("--json", default="")
-    args = ap.parse_args()
-    only = [s for s in args.only.split(",") if s]
-
-    L = pkg.load("bf16")          # raises LibraryMissing when the HIP library has not been built
-    L.llmk_init(0)
+def run_cases(L, reps=20, only=(), emit=print):
+    """Runs every case (or those whose tag contains one of `only`) on the loaded library L and returns the list of
+    per-kernel records. `emit` receives the printed lines (None: silent)."""
+    only = list(only)
     dev = "cuda"
     p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
     g = torch.Generator(device=dev); g.manual_seed(1234)
@@ -57,7 +51,7 @@ def main():
         """-> {family: (list of ms per rep, flops per rep, bytes per rep, launches per rep)}"""
         out = {}
         fn(); torch.cuda.synchronize()                        # warm-up (workspace growth, attribute setting)
-        for _ in range(args.reps):
+        for _ in range(reps):
             if prepare: prepare()
             flush_buf.zero_(); torch.cuda.synchronize()
             L.llmk_profile_reset(); L.llmk_profile_enable(1)
@@ -79,8 +73,8 @@ def main():
                 rate, unit, frac = flops / med * 1e-9, "TFLOP/s", flops / med * 1e-9 / PEAK_TFLOPS
             else:
                 rate, unit, frac = nbytes / med * 1e-6, "GB/s", nbytes / med * 1e-6 / PEAK_GBS
-            print(f"{case:34s} {fam:26s} x{ncalls:<2d} median {med:8.4f} ms  min {mn:8.4f} ms  {rate:9.1f} {unit:8s} {100 * frac:5.1f} % of {'MFMA' if mfma else 'HBM'} peak",
-                  flush=True)
+            if emit:
+                emit(f"{case:34s} {fam:26s} x{ncalls:<2d} median {med:8.4f} ms  min {mn:8.4f} ms  {rate:9.1f} {unit:8s} {100 * frac:5.1f} % of {'MFMA' if mfma else 'HBM'} peak")
             results.append({"case": case, "kernel": fam, "launches": ncalls, "median_ms": med, "min_ms": mn, "rate": rate, "unit": unit,
                             "bound": "mfma" if mfma else "hbm", "frac": frac, "flops": flops, "bytes": nbytes})
 
@@ -108,6 +102,11 @@ def main():
             scratch = torch.empty(max(L.llmk_matmul_backward_bias_scratch_floats(OC), 1), device=dev, dtype=torch.float32)
             report(f"matmul_backward {nm} K={K} OC={OC}",
                    measure(lambda: L.llmk_matmul_backward(p(dinp), p(dw), p(dbias), p(dout), p(inp), p(w), p(scratch), B, T, K, OC, None, None, 0)))
+            if nm == "fcproj":                                 # the dinp GEMM with GELU backward in its epilogue (gelu_fusion 2)
+                pre = randn(N, K)
+                report(f"matmul_backward+dgelu {nm} K={K} OC={OC}",
+                       measure(lambda: L.llmk_matmul_backward(p(dinp), p(dw), p(dbias), p(dout), p(inp), p(w), p(scratch), B, T, K, OC, None, p(pre), 2)))
+                del pre
             del inp, w, out_t, dout, dinp, dw, scratch
             torch.cuda.empty_cache()
 
@@ -186,6 +185,21 @@ def main():
         report("attention_backward B64 NH12 T1024 hs64",
                measure(lambda: L.llmk_attention_backward(p(dqkv), p(dout), p(qkv), p(o), p(stats), B, T, NH, Cc, None)))
 
+    L.llmk_profile_reset()
+    del flush_buf
+    torch.cuda.empty_cache()
+    return results
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--reps", type=int, default=20)
+    ap.add_argument("--only", default="")
+    ap.add_argument("--json", default="")
+    args = ap.parse_args()
+    L = pkg.load("bf16")          # raises LibraryMissing when the HIP library has not been built
+    L.llmk_init(0)
+    results = run_cases(L, args.reps, [s for s in args.only.split(",") if s], lambda line: print(line, flush=True))
     if args.json:
         with open(args.json, "w") as f:
             json.dump({"reps": args.reps, "peak_tflops": PEAK_TFLOPS, "peak_gbs": PEAK_GBS, "results": results}, f, indent=1)
