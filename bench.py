@@ -152,12 +152,12 @@ class SclkSampler:
 
 
 def default_headline(args):
-    return (args.batch, args.seq, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 2)
+    return (args.batch, args.seq, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 3)
 
 
 def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, kernel_events, lr=6e-4):
     """Builds the model, runs warmup + steps training steps on one synthetic batch, returns the result fields."""
-    default_workload = (B, T, model, recompute, gelu_fusion) == (64, 1024, "d12", 0, 2)
+    default_workload = (B, T, model, recompute, gelu_fusion) == (64, 1024, "d12", 0, 3)
     h = L.gpt2_create()
     L.gpt2_set_options(h, 1, recompute, gelu_fusion)
     L.gpt2_build_from_descriptor(h, model.encode())
@@ -274,7 +274,9 @@ def main():
     ap.add_argument("--seq", type=int, default=1024)
     ap.add_argument("--model", default="d12")
     ap.add_argument("--recompute", type=int, default=0)   # the reference's 124M recipe runs with -r 0 (scripts/run_gpt2_124M.sh)
-    ap.add_argument("--gelu-fusion", type=int, default=2)
+    # 3: GELU in both GEMM epilogues with gelu'(pre-activation) kept for the backward one (this library's own level; the
+    # reference's highest is 2, which --gelu-fusion 2 runs)
+    ap.add_argument("--gelu-fusion", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
@@ -349,7 +351,7 @@ def main():
         # own recipe (scripts/run_gpt2_350M.sh:29-34: -b 64; scripts/run_gpt2_1558M.sh:27-33 has -b 16). No recomputation
         # (-r 0) and the learning rates of those recipes.
         for model, b, lr in (("d24", 32, 3e-4), ("d48", 16, 6e-4), ("d24", 64, 3e-4)):
-            r = run_workload(L, torch, model, b, 1024, 0, 2, 3, 2, False, lr=lr)
+            r = run_workload(L, torch, model, b, 1024, 0, args.gelu_fusion, 3, 2, False, lr=lr)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
                                                               "loss_first", "loss_last", "losses")})
     if default_headline(args) and not args.no_microbench:

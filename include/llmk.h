@@ -127,7 +127,11 @@ size_t llmk_layernorm_backward_scratch_floats(int C);
 
 /* matmul_forward_cublaslt, llmc/matmul.cuh:231. out[B*T,OC] = inp[B*T,C] . weight[OC,C]^T + bias[OC].
  * bias may be NULL. If pre_gelu != NULL: pre_gelu receives the pre-activation and out = gelu(pre_gelu)
- * (gelu_fusion >= 1: in the GEMM epilogue; < 1: separate gelu kernel). */
+ * (gelu_fusion >= 1: in the GEMM epilogue; < 1: separate gelu kernel).
+ * gelu_fusion 3 has no counterpart in the reference (its levels are 0-2, train_gpt2.cu:1419-1470): pre_gelu then
+ * receives gelu'(pre-activation), rounded to the storage type, instead of the pre-activation, for a backward pass that
+ * only multiplies by it (llmk_matmul_backward with gelu_fusion 3). For callers that keep the tensor for nothing else,
+ * i.e. that do not recompute gelu from it. out is the same bits as with gelu_fusion 1 and 2. */
 void llmk_matmul_forward(void* out, const void* inp, const void* weight, const void* bias, int B, int T, int C,
                          int OC, void* stream, void* pre_gelu, int gelu_fusion);
 
@@ -136,6 +140,8 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
  *   dinp[B*T,C]  = dout . weight                 (then *= gelu'(pre_gelu) when pre_gelu != NULL;
  *                                                 gelu_fusion >= 2: in the epilogue, else separate kernel)
  *   dweight[OC,C] += dout^T . inp
+ * gelu_fusion 3: pre_gelu holds gelu'(pre-activation) as llmk_matmul_forward(.., gelu_fusion 3) left it, and dinp is
+ * the product of the rounded dout . weight with that stored value, rounded once more.
  * dbias_buffer: device fp32 scratch, >= llmk_matmul_backward_bias_scratch_floats(OC) floats
  * (may be NULL when dbias == NULL). */
 void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
@@ -200,6 +206,12 @@ void llmk_attention_backward_static(void* dqkvr, const void* dout, const void* q
                                     int B, int T, int NH, int C, void* stream);
 
 /* ---- gelu (llmc/gelu.cuh) ----------------------------------------------------------------- */
+
+/* The two halves of gelu_fusion 3 as passes of their own (what llmk_matmul_forward / llmk_matmul_backward run for shapes
+ * their fused epilogues do not take); no counterpart in the reference. out = gelu(inp_to_grad), then inp_to_grad =
+ * gelu'(inp_to_grad) in place; d_in_out *= grad. */
+void llmk_gelu_forward_keep_grad(void* out, void* inp_to_grad, int N, void* stream);
+void llmk_gelu_backward_from_grad(void* d_in_out, const void* grad, int N, void* stream);
 
 /* gelu_forward, llmc/gelu.cuh:50 */
 void llmk_gelu_forward(void* out, const void* inp, int N, void* stream);

@@ -22,7 +22,9 @@ typedef struct LLMK_GPT2 LLMK_GPT2;
  * rng_state=13371337. */
 LLMK_GPT2* gpt2_create(void);
 /* options that the reference sets on the struct before gpt2_allocate_state (train_gpt2.cu:1578-1581):
- * use_master_weights 0|1, recompute 0|1|2, gelu_fusion 0|1|2; negative = leave unchanged */
+ * use_master_weights 0|1, recompute 0|1|2, gelu_fusion 0|1|2; negative = leave unchanged.
+ * gelu_fusion 3 (this library's own, see llmk_matmul_forward): the fch tensor keeps gelu'(pre-activation) for the backward
+ * epilogue instead of the pre-activation; with recompute >= 1, which needs the pre-activation again, it runs as 2. */
 void gpt2_set_options(LLMK_GPT2* m, int use_master_weights, int recompute, int gelu_fusion);
 
 /* gpt_build_from_descriptor, train_gpt2.cu:562: "d12", "gpt2:d48", "gpt3:c768"; mt19937 seed 42 */

@@ -42,6 +42,8 @@ KERNEL_ABI = {
     "llmk_clear_error": (None, []),
     "llmk_profile_enable": (None, [i32]),
     "llmk_matmul_backward_split_mode": (None, [i32]),
+    "llmk_gelu_forward_keep_grad": (None, [vp, vp, i32, vp]),
+    "llmk_gelu_backward_from_grad": (None, [vp, vp, i32, vp]),
     "llmk_matmul_backward_last_split": (None, [ip, ip]),
     "llmk_matmul_backward_workspace_bytes": (sz, [i32, i32, i32, i32]),
     "llmk_attention_backward_workspace_bytes": (sz, [i32, i32, i32]),

@@ -40,3 +40,18 @@ __device__ __forceinline__ float gelu_grad_f(float x) {
     return fmaf(x * s, (1.0f - s) * du2, s);
 }
 #endif
+// gelu(x) and gelu'(x) together, each the same bits as the function of its own: for a forward pass that leaves the
+// derivative behind for the backward pass (gelu_fusion 3) instead of the pre-activation.
+#if defined(LLMK_FP32)
+__device__ __forceinline__ float gelu_with_grad_f(float x, float& grad) { grad = gelu_grad_f(x); return gelu_f(x); }
+#else
+__device__ __forceinline__ float gelu_with_grad_f(float x, float& grad) {
+    const float k2 = 2.0f * 0.7978845608028654f;
+    const float x2 = x * x;
+    const float s = gelu_sigmoid(x, x2);                                    // shared: the one exp2 and the one reciprocal
+    const float xs = x * s;
+    const float du2 = fmaf(x2, k2 * 3.0f * 0.044715f, k2);
+    grad = fmaf(xs, (1.0f - s) * du2, s);
+    return xs;
+}
+#endif

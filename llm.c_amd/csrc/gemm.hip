@@ -696,7 +696,20 @@ void llmk_matmul_forward(void* out, const void* inp, const void* weight, const v
     const bool gelu_in_gemm = pre_gelu && gelu_fusion >= 1;            // then the kernel writes two (M, OC) tensors
     llmk::ProfScope prof(gelu_in_gemm ? "gemm_nt_gelu" : "gemm_nt", 2.0 * M * (double)OC * C,
                          ((double)M * C + (double)OC * C + (gelu_in_gemm ? 2.0 : 1.0) * M * OC) * sizeof(floatX), st);
-    if (pre_gelu && gelu_fusion >= 1) {
+    if (pre_gelu && gelu_fusion >= 3) {
+        // pre_gelu receives gelu'(pre-activation): in the direct-to-LDS kernel's epilogue, else by a pass of its own
+        g.C = (floatX*)out; g.aux = (floatX*)pre_gelu;
+#if !defined(LLMK_FP32)
+        if (big && pipelined_ok(g)) {
+            launch_pipelined_cfg<256, 256, 2, 4, false, false, EPI_BIAS_GELU_D>(g, 1, st);
+            return;
+        }
+#endif
+        g.C = (floatX*)pre_gelu; g.aux = nullptr;
+        launch_best<false, false, EPI_BIAS>(g, 1, big, st);
+        if (prof.on) { llmk::prof_end(st); prof.on = false; }
+        llmk_gelu_forward_keep_grad(out, pre_gelu, M * OC, stream);
+    } else if (pre_gelu && gelu_fusion >= 1) {
         g.C = (floatX*)out; g.aux = (floatX*)pre_gelu;
         launch_best<false, false, EPI_BIAS_GELU>(g, 1, big, st);
     } else if (pre_gelu) {
@@ -799,8 +812,9 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
         g.M = M; g.N = C; g.K = OC; g.lda = OC; g.ldb = C; g.ldc = C;
         g.k_per_split = CEIL_DIV(OC, K_STEP) * K_STEP;
         const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(C, BIG_TILE) >= (size_t)num_cu;
+        const bool stored_grad = pre_gelu && gelu_fusion >= 3;   // pre_gelu holds gelu'(pre-activation), see llmk_matmul_forward
 #if defined(LLMK_FP32)
-        const bool fused = pre_gelu && gelu_fusion >= 2;
+        const bool fused = pre_gelu && gelu_fusion >= 2 && !stored_grad;
 #else
         // bf16: gelu' goes into the epilogue of the direct-to-LDS kernel (big tiles only); the bias gradient of the layer
         // below then comes out of its weight-gradient GEMM, and no elementwise pass over (B,T,4C) is left
@@ -815,13 +829,17 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
 #if defined(LLMK_FP32)
                 launch_best<false, true, EPI_DGELU>(g, 1, big, st);
 #else
-                launch_pipelined_cfg<256, 256, 2, 4, false, true, EPI_DGELU>(g, 1, st);
+                if (stored_grad) launch_pipelined_cfg<256, 256, 2, 4, false, true, EPI_DGELU_D>(g, 1, st);
+                else launch_pipelined_cfg<256, 256, 2, 4, false, true, EPI_DGELU>(g, 1, st);
 #endif
             } else {
                 launch_best<false, true, EPI_STORE>(g, 1, big, st);
             }
         }
-        if (pre_gelu && !fused) llmk_gelu_backward_inplace(dinp, pre_gelu, M * C, stream);
+        if (pre_gelu && !fused) {
+            if (stored_grad) llmk_gelu_backward_from_grad(dinp, pre_gelu, M * C, stream);
+            else llmk_gelu_backward_inplace(dinp, pre_gelu, M * C, stream);
+        }
     }
 
     // (3) dW[OC,C] += dout^T . inp   (A(m=oc,k=row) stored [k][m], B(n=c,k=row) stored [k][n])

@@ -43,7 +43,13 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 
 // EPI_PARTIAL_ROWSUM: EPI_PARTIAL plus, per row m of the output, the sum over the split's K range of A(m, k): with
 // A = dout^T that is the bias gradient, taken from the operand fragments the matrix cores are being fed anyway.
-enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5, EPI_PARTIAL_ROWSUM = 6 };
+// EPI_BIAS_GELU_D / EPI_DGELU_D (gelu_fusion 3): the forward epilogue leaves gelu'(pre-activation) in the second output
+// instead of the pre-activation, and the backward epilogue multiplies by that stored value: the exponential, the
+// reciprocal and nine of the thirteen vector operations per element move out of the backward epilogue, four into the forward one.
+enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5, EPI_PARTIAL_ROWSUM = 6,
+           EPI_BIAS_GELU_D = 7, EPI_DGELU_D = 8 };
+constexpr bool epi_gelu_fwd(int e) { return e == EPI_BIAS_GELU || e == EPI_BIAS_GELU_D; }
+constexpr bool epi_gelu_bwd(int e) { return e == EPI_DGELU || e == EPI_DGELU_D; }
 
 struct GemmArgs {
     const floatX* A;
@@ -52,7 +58,7 @@ struct GemmArgs {
     int M, N, K;          // C[M][N] = sum_k A(m,k) * B(n,k)
     int lda, ldb, ldc;    // leading dimensions of the stored matrices, in elements
     const floatX* bias;   // [N] or nullptr                         (EPI_BIAS*)
-    floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU)
+    floatX* aux;          // pre-GELU output (EPI_BIAS_GELU) / pre-GELU input (EPI_DGELU); gelu' of it for the _D pair
     float* partial;       // [splits][M][N] fp32                    (EPI_PARTIAL*)
     float* rowsum;        // [splits * WGN][M] fp32 (WGN: column waves of the tile configuration)  (EPI_PARTIAL_ROWSUM)
     int k_per_split;      // multiple of the K block
@@ -390,7 +396,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     // everything but the N youngest has landed. The stages of a tile are requested one at a time, so the only
     // younger operations a wait ever has to allow are the second stage of the tile's prologue and the previous
     // tile's output stores (NS_EPI per wave when every lane stored, which holds for interior tiles).
-    constexpr int NS_EPI = TM * PASSES_OF_EPI * 4 * (EPI == EPI_BIAS_GELU ? 2 : 1);
+    constexpr int NS_EPI = TM * PASSES_OF_EPI * 4 * (epi_gelu_fwd(EPI) ? 2 : 1);
     static_assert(CPW + NS_EPI <= 63, "vmcnt is a 6-bit counter");
 
     int it = 0;
@@ -409,14 +415,14 @@ gemm_pipelined_kernel(GemmArgs g) {
     // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
     constexpr bool F32OUT = (IS_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
     constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
-    constexpr bool EPI_READS = (EPI == EPI_ACCUM || EPI == EPI_DGELU);
+    constexpr bool EPI_READS = (EPI == EPI_ACCUM || epi_gelu_bwd(EPI));
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
     // GELU backward: the pre-activation values of the 16 bytes each lane stores per (block, pass, quarter), as it stores them
-    u32x4 pre_act[EPI == EPI_DGELU ? TM : 1][EPI == EPI_DGELU ? PASSES : 1][4];
+    u32x4 pre_act[epi_gelu_bwd(EPI) ? TM : 1][epi_gelu_bwd(EPI) ? PASSES : 1][4];
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
         if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
-        if constexpr (EPI == EPI_DGELU) {
+        if constexpr (epi_gelu_bwd(EPI)) {
 #pragma unroll
             for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
@@ -449,7 +455,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     // last-but-one stage ended with a wait for everything) until the wave requests the next tile's first stage, which
     // these kernels do only after claiming the bias (bias_ready), half-way through the last stage. Tiles that reach past N take plain
     // loads in the epilogue instead (the columns are tested there).
-    constexpr bool HAS_BIAS = (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU);
+    constexpr bool HAS_BIAS = (EPI == EPI_BIAS || epi_gelu_fwd(EPI));
     bf16x4 biasv[HAS_BIAS ? TN : 1][4];
     bool bias_fast = false;
     auto request_bias = [&](int n0) {
@@ -618,7 +624,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                                 const bf16x4 b4 = biasv[HAS_BIAS ? j : 0][q];
 #pragma unroll
                                 for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
-                            } else if (EPI == EPI_BIAS || EPI == EPI_BIAS_GELU) {
+                            } else if (HAS_BIAS) {
                                 if (g.bias) {
                                     const int n = wn0 + nl;
                                     if (n < g.N) {
@@ -674,12 +680,24 @@ gemm_pipelined_kernel(GemmArgs g) {
 #pragma unroll
                                     for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
                                     st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
-                                } else if (EPI == EPI_DGELU) {
-                                    // the product of the rounded gradient and gelu'(pre), as gelu_backward_inplace forms it
-                                    union { u32x4 u; bf16x8 h; } pa;
-                                    pa.u = pre_act[EPI == EPI_DGELU ? i : 0][EPI == EPI_DGELU ? pass : 0][t];
+                                } else if (EPI == EPI_BIAS_GELU_D) {
+                                    union { u32x4 u; bf16x8 h; } d;
 #pragma unroll
-                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)(gelu_grad_f((float)pa.h[e]) * (float)x.h[e]);
+                                    for (int e = 0; e < 8; e++) {
+                                        float gr;
+                                        y.h[e] = (__bf16)gelu_with_grad_f((float)x.h[e], gr);
+                                        d.h[e] = (__bf16)gr;
+                                    }
+                                    st_out(reinterpret_cast<u32x4*>(g.aux + o), d.u);
+                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                } else if (epi_gelu_bwd(EPI)) {
+                                    // the product of the rounded gradient and gelu'(pre), as gelu_backward_inplace forms it
+                                    // (EPI_DGELU_D: gelu'(pre) is what was stored)
+                                    union { u32x4 u; bf16x8 h; } pa;
+                                    pa.u = pre_act[epi_gelu_bwd(EPI) ? i : 0][epi_gelu_bwd(EPI) ? pass : 0][t];
+#pragma unroll
+                                    for (int e = 0; e < 8; e++)
+                                        y.h[e] = (__bf16)((EPI == EPI_DGELU_D ? (float)pa.h[e] : gelu_grad_f((float)pa.h[e])) * (float)x.h[e]);
                                     st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
                                 } else {
                                     st_out(reinterpret_cast<u32x4*>(g.C + o), x.u);

@@ -327,6 +327,10 @@ LLMK_GPT2* gpt2_create(void) {
     return m;
 }
 
+// gelu_fusion 3 leaves gelu'(fch) in the fch tensor; recomputing fch_gelu in the backward pass (recompute >= 1) needs
+// fch itself, so those runs take level 2
+static int gelu_fusion_in_use(const LLMK_GPT2* m) { return (m->gelu_fusion >= 3 && m->recompute >= 1) ? 2 : m->gelu_fusion; }
+
 void gpt2_set_options(LLMK_GPT2* m, int use_master_weights, int recompute, int gelu_fusion) {
     if (use_master_weights >= 0) m->use_master_weights = use_master_weights;
     if (recompute >= 0) m->recompute = recompute;
@@ -459,7 +463,7 @@ void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T) {
         llmk_attention_forward(l_atty, l_att, l_qkvr, (int)B, (int)T, (int)NH, (int)C, st);
         llmk_matmul_forward(scratch, l_atty, l_attprojw, l_attprojb, (int)B, (int)T, (int)C, (int)C, st, nullptr, 1);
         llmk_fused_residual_forward5(l_residual2, l_ln2, l_ln2_mean, l_ln2_rstd, residual, scratch, l_ln2w, l_ln2b, (int)(B * T), (int)C, st);
-        llmk_matmul_forward(l_fch_gelu, l_ln2, l_fcw, l_fcb, (int)B, (int)T, (int)C, (int)(4 * C), st, l_fch, m->gelu_fusion);
+        llmk_matmul_forward(l_fch_gelu, l_ln2, l_fcw, l_fcb, (int)B, (int)T, (int)C, (int)(4 * C), st, l_fch, gelu_fusion_in_use(m));
         llmk_matmul_forward(scratch, l_fch_gelu, l_fcprojw, l_fcprojb, (int)B, (int)T, (int)(4 * C), (int)C, st, nullptr, 1);
         if (l + 1 != L) {
             xptr n_ln1 = R < 2 ? off(a.ln1, (l + 1) * B * T * C, X) : a.lnf;
@@ -571,7 +575,7 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
         if (R >= 1) llmk_gelu_forward(l_fch_gelu, l_fch_pre_gelu, (int)(B * T * 4 * C), st);
         // with gelu_fusion 2 the GELU backward is the epilogue of this GEMM's dinp; the bias gradient of the fc layer, whose
         // dout that produces, comes out of the fc weight-gradient GEMM below
-        llmk_matmul_backward(dl_bt4c, dl_fcprojw, dl_fcprojb, dresidual, l_fch_gelu, l_fcprojw, scratchF, (int)B, (int)T, (int)(4 * C), (int)C, st, l_fch_pre_gelu, m->gelu_fusion);
+        llmk_matmul_backward(dl_bt4c, dl_fcprojw, dl_fcprojb, dresidual, l_fch_gelu, l_fcprojw, scratchF, (int)B, (int)T, (int)(4 * C), (int)C, st, l_fch_pre_gelu, gelu_fusion_in_use(m));
         if (R >= 2) llmk_layernorm_forward(l_ln2, l_ln2_mean, l_ln2_rstd, l_residual2, l_ln2w, l_ln2b, (int)B, (int)T, (int)C, st);
         llmk_matmul_backward(dl_btc, dl_fcw, dl_fcb, dl_bt4c, l_ln2, l_fcw, scratchF, (int)B, (int)T, (int)C, (int)(4 * C), st, nullptr, 1);
         llmk_layernorm_backward(dresidual, dl_ln2w, dl_ln2b, scratchF, dl_btc, l_residual2, l_ln2w, l_ln2_mean, l_ln2_rstd, (int)B, (int)T, (int)C, st);

@@ -50,7 +50,7 @@ namespace {
             "  -h <int>    hellaswag eval run? (default = 0)\n"
             "  -a <int>    overfit a single batch? 0/1. useful for debugging\n"
             "  -w <int>    keep f32 copy of weights for the optimizer? (default: 1)\n"
-            "  -ge <int>   gelu fusion: 0=none, 1=forward, 2=forward+backward (default: 2)\n"
+            "  -ge <int>   gelu fusion: 0=none, 1=forward, 2=forward+backward, 3=2 with gelu' kept for backward (with -r 0) (default: 2)\n"
             "  -r <int>    recompute: less memory but less speed. (default = 1), 0|1|2 = none,gelu,gelu+ln\n"
             "  -f, -z, -pn, -pr, -pg, -pi, -pf, -ps: accepted for compatibility; one process only\n");
     exit(EXIT_FAILURE);

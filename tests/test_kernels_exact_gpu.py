@@ -114,6 +114,42 @@ def test_forward_projection_with_gelu_epilogue(C, OC):
     G.check_no_error(L)
 
 
+@pytest.mark.parametrize("C,OC", [(768, 3072), (1024, 4096), (1600, 6400)])
+def test_gelu_fusion_3_epilogues_at_the_training_shapes(C, OC):
+    """The fc layer forward with gelu_fusion 3 and the fcproj layer's dinp that consumes it: the activated output is the
+    same bits as with fusion 2, the second output is the library's own GELU derivative of the exact pre-activation
+    (what llmk_gelu_backward_inplace makes of a tensor of ones), and dinp is the exact product, rounded, times that
+    stored value, rounded once (a product of two bf16 values is exact in fp32)."""
+    import torch
+    L = G.lib("bf16")
+    M = N_ROWS if OC <= 3072 else N_ROWS // 4
+    x, w, b = ints((M, C), 4), ints((OC, C), 5, scale=1.0 / 64), ints((OC,), 6, -8, 8, scale=1.0 / 8)
+    out = torch.zeros((M, OC), dtype=torch.bfloat16, device="cuda")
+    grad = torch.zeros((M, OC), dtype=torch.bfloat16, device="cuda")
+    L.llmk_matmul_forward(G.ptr(out), G.ptr(x), G.ptr(w), G.ptr(b), 1, M, C, OC, None, G.ptr(grad), 3)
+    G.sync()
+    pre = (exact_nt(x, w) + b.float()).to(torch.bfloat16)
+    want = torch.zeros_like(out)
+    L.llmk_gelu_forward(G.ptr(want), G.ptr(pre), M * OC, None)
+    want_grad = torch.ones_like(out)
+    L.llmk_gelu_backward_inplace(G.ptr(want_grad), G.ptr(pre), M * OC, None)
+    G.sync()
+    assert torch.equal(out, want)
+    assert torch.equal(grad, want_grad)
+    del pre, want, want_grad, out
+    # backward: dinp (M, OC) = (dout (M, C) . w2 (C, OC)) * stored derivative
+    g, w2 = ints((M, C), 14, -2, 2), ints((C, OC), 13)
+    dx = torch.zeros((M, OC), dtype=torch.bfloat16, device="cuda")
+    dw = torch.zeros((C, OC), dtype=torch.bfloat16, device="cuda")
+    inp = ints((M, OC), 12, -2, 2)
+    L.llmk_matmul_backward(G.ptr(dx), G.ptr(dw), None, G.ptr(g), G.ptr(inp), G.ptr(w2), None, 1, M, OC, C, None, G.ptr(grad), 3)
+    G.sync()
+    lin = exact_nt(g, w2.t().contiguous()).to(torch.bfloat16)
+    assert torch.equal(dx, (lin.float() * grad.float()).to(torch.bfloat16))
+    assert_same_bits(dw, exact_tn(g, inp), "dweight")
+    G.check_no_error(L)
+
+
 @pytest.mark.parametrize("split_mode", [0, 1])
 @pytest.mark.parametrize("C,OC", LAYER_SHAPES + [(1600, 1600), (1600, 6400)])
 def test_backward_projection_is_the_integer_product(C, OC, split_mode):

@@ -374,6 +374,43 @@ def test_matmul_backward_gelu(precision, fusion, M, Cc, OC):
     G.check_no_error(L)
 
 
+@pytest.mark.parametrize("precision", PRECS)
+@pytest.mark.parametrize("M,Cc,OC", [(320, 128, 512),        # few tiles: the two halves as passes of their own
+                                     (8192, 512, 2048),      # a tile per CU and more: both in GEMM epilogues (bf16)
+                                     (8448, 192, 2056)])     # ... with ragged last tiles in both directions
+def test_gelu_fusion_3_keeps_the_derivative_for_backward(precision, M, Cc, OC):
+    """gelu_fusion 3 (no counterpart in the reference): the forward pass leaves gelu'(pre-activation) where levels 0-2
+    leave the pre-activation, and the backward pass multiplies by it. Against the oracle's GELU forward and backward
+    (train_gpt2.c:407-433) applied to the pre-activation that level 2 reports: the output to the usual bound (it is
+    the same bits as level 2's), the stored derivative to one rounding of the storage type, and dinp of the projection
+    that follows (its contraction length is the fc width OC) to the bound of test_matmul_backward_gelu."""
+    import torch
+    L = G.lib(precision)
+    x, w, b = G.rounded(rnd((M, Cc), 0), precision), G.rounded(rnd((OC, Cc), 1, 0.1), precision), G.rounded(rnd(OC, 2), precision)
+    out2, pre = run_matmul_forward(L, precision, x, w, b, True, 2)
+    out3, grad = run_matmul_forward(L, precision, x, w, b, True, 3)
+    assert np.array_equal(out2, out3)
+    ones = np.ones(pre.size, np.float32)
+    want_grad = np.zeros(pre.size, np.float32)
+    ol.cref().cref_gelu_backward(want_grad, np.ascontiguousarray(pre).reshape(-1), ones, pre.size)
+    close(grad.reshape(-1), want_grad, **tol(precision, 2e-5, bf16_rel=1.0 / 128, bf16_atol=1e-2), what="stored gelu'")
+    # backward of the projection that consumes gelu(pre): dinp (M, OC) = (dout (M, Cc2) . w2 (Cc2, OC)) * gelu'(pre)
+    Cc2 = 128
+    g, w2 = G.rounded(rnd((M, Cc2), 5), precision), G.rounded(rnd((Cc2, OC), 6, 0.1), precision)
+    lin = G.rounded((g.astype(np.float64) @ w2.astype(np.float64)).astype(np.float32), precision)
+    ref = np.zeros((M, OC), np.float32)
+    ol.cref().cref_gelu_backward(ref.reshape(-1), np.ascontiguousarray(pre).reshape(-1), lin.reshape(-1), M * OC)
+    d_dx, d_dw = G.dev(np.zeros((M, OC), np.float32), precision), G.dev(np.zeros((Cc2, OC), np.float32), precision)
+    d_g, d_in, d_w2, d_grad = G.dev(g, precision), G.dev(out3, precision), G.dev(w2, precision), G.dev(grad, precision)
+    L.llmk_matmul_backward(G.ptr(d_dx), G.ptr(d_dw), None, G.ptr(d_g), G.ptr(d_in), G.ptr(d_w2), None, 1, M, OC, Cc2, None,
+                           G.ptr(d_grad), 3)
+    got = G.host(d_dx)
+    close(got, ref, **tol(precision, 1e-4, bf16_rel=1.0 / 32, bf16_atol=3e-2))
+    # three bf16 roundings (the product, the derivative, the result) instead of level 2's two
+    assert rel_fro(got, ref) < (1e-5 if precision == "fp32" else 5e-3), rel_fro(got, ref)
+    G.check_no_error(L)
+
+
 # ------------------------------------------------------------------------------------------------
 def attention_case(precision, B, T, NH, seed=0, hs=64):
     Cc = NH * hs
