@@ -7,6 +7,7 @@ Makefile:232-244). hipcc cross-compiles for gfx950, so this also runs on a machi
 
     python llm.c_amd/build.py            # both precisions
     python llm.c_amd/build.py bf16       # one
+    python llm.c_amd/build.py --variant noloads -DLLMK_GEMM_ABL=1   # a measurement build beside the product library
 """
 import os
 import subprocess
@@ -48,9 +49,18 @@ def _run(cmd):
     return out
 
 
-def build(precisions=("bf16", "fp32"), jobs=8, verbose=False):
+def variant_dir(name):
+    return os.path.join(LIBDIR, "variants", name)
+
+
+def build(precisions=("bf16", "fp32"), jobs=8, verbose=False, variant=None, defines=()):
+    """variant: build lib/variants/<variant>/libllmk_<precision>.so with the extra -D defines instead of the product
+    library (measurement builds for microbench.py --variant: ablation switches of the kernels; nothing loads them by
+    default and they are not part of what tests, bench.py or the trainer run)."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     os.makedirs(LIBDIR, exist_ok=True)
+    if variant:
+        return _build_variant(hipcc, precisions, variant, list(defines), jobs, verbose)
     tasks = []
     objs = {p: [] for p in precisions}
     for p in precisions:
@@ -78,7 +88,40 @@ def build(precisions=("bf16", "fp32"), jobs=8, verbose=False):
     return [lib_path(p) for p in precisions]
 
 
+def _build_variant(hipcc, precisions, variant, defines, jobs, verbose):
+    out = []
+    for p in precisions:
+        od = os.path.join(OBJDIR, f"{p}_{variant}")
+        os.makedirs(od, exist_ok=True)
+        os.makedirs(variant_dir(variant), exist_ok=True)
+        tasks, objs = [], []
+        for src in KERNEL_SOURCES:
+            o = os.path.join(od, src + ".o")
+            objs.append(o)
+            tasks.append([hipcc, *COMMON, *PREC_DEFS[p], *defines, "-c", os.path.join(CSRC, src), "-o", o])
+        for src in DRIVER_SOURCES:
+            o = os.path.join(od, src + ".o")
+            objs.append(o)
+            tasks.append([hipcc, *COMMON, *PREC_DEFS[p], *defines, "-x", "hip", "-c", os.path.join(DRIVER, src), "-o", o])
+        with ThreadPoolExecutor(max_workers=jobs) as ex:
+            for text in ex.map(_run, tasks):
+                if verbose and text.strip():
+                    print(text)
+        path = os.path.join(variant_dir(variant), f"libllmk_{p}.so")
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", path, *objs])
+        out.append(path)
+    return out
+
+
 if __name__ == "__main__":
-    precs = tuple(sys.argv[1:]) or ("bf16", "fp32")
-    for path in build(precs, verbose=True):
+    import argparse
+    ap = argparse.ArgumentParser()
+    ap.add_argument("precisions", nargs="*", default=[])
+    ap.add_argument("--variant", default=None, help="build lib/variants/NAME/ with the given -D switches instead of the product library")
+    args, extra = ap.parse_known_args()
+    defines = [a for a in extra if a.startswith("-D")]
+    if [a for a in extra if not a.startswith("-D")]:
+        ap.error("unknown arguments: " + " ".join(a for a in extra if not a.startswith("-D")))
+    precs = tuple(args.precisions) or (("bf16",) if args.variant else ("bf16", "fp32"))
+    for path in build(precs, verbose=True, variant=args.variant, defines=defines):
         print(path)

@@ -79,6 +79,13 @@ constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 #ifndef LLMK_TR_ASM_MIXED
 #define LLMK_TR_ASM_MIXED 0
 #endif
+// Timing-only ablations of the kernel's parts, for llm.c_amd/microbench.py --variant (python llm.c_amd/build.py --variant
+// NAME -DLLMK_GEMM_ABL=bits builds a library beside the product one; results of such a build are wrong by design):
+//   1  no global -> LDS stage loads after a workgroup's first two stages     2  no matrix instructions
+//   4  no fragment reads from LDS                                             8  no epilogue (strip passes and stores)
+#ifndef LLMK_GEMM_ABL
+#define LLMK_GEMM_ABL 0
+#endif
 constexpr int PBK = 64;                 // K per stage
 constexpr int STAGES = 2;               // operand buffers: one being multiplied, one being filled
 constexpr int KGRAN = PBK;              // K (and the K range of a split) must be a multiple of this
@@ -272,7 +279,9 @@ gemm_pipelined_kernel(GemmArgs g) {
     // The loads are issued from inline asm, M0 (the LDS destination) included: when the compiler knows of a
     // direct-to-LDS load in flight it makes every later LDS read it can see wait for ALL loads, e.g. the epilogue's
     // strip reads for the next tile's first stages. All waiting for these loads is explicit (wait_vmcnt).
+    bool abl_loads_on = true;          // (LLMK_GEMM_ABL & 1: switched off after the first two stage requests)
     auto issue_from = [&](const char* const (&tb)[2], int st, int buf) {
+        if ((LLMK_GEMM_ABL & 1) && !abl_loads_on) return;
         const unsigned stage = lds0 + buf * STAGE;
         const unsigned long long pa = (unsigned long long)(size_t)(tb[0] + (size_t)st * stage_step[0]);
         const unsigned long long pb = (unsigned long long)(size_t)(tb[1] + (size_t)st * stage_step[1]);
@@ -330,6 +339,13 @@ gemm_pipelined_kernel(GemmArgs g) {
     // fragments of the 16-wide K step S of the buffer at byte offset bufoff
     auto read_frags = [&](unsigned bufoff, auto sc, bf16x8 (&fa)[TM], bf16x8 (&fb)[TN]) {
         constexpr int S = decltype(sc)::value;
+        if (LLMK_GEMM_ABL & 4) {                                  // the registers count as rewritten, nothing is read
+#pragma unroll
+            for (int i = 0; i < TM; i++) asm volatile("" : "+v"(fa[i]));
+#pragma unroll
+            for (int j = 0; j < TN; j++) asm volatile("" : "+v"(fb[j]));
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++) {
             if constexpr (A_T) fa[i] = frag_t(abase[i] + bufoff, std::integral_constant<int, S * 16 * BM * 2>{}, std::integral_constant<int, (S * 16 + 4) * BM * 2>{});
@@ -374,6 +390,13 @@ gemm_pipelined_kernel(GemmArgs g) {
     float rsum[ROWSUM ? TM : 1];
     int rowsum_step = -1;                  // the step of a stage this wave sums in the current tile, or none
     auto mma = [&](const bf16x8 (&fa)[TM], const bf16x8 (&fb)[TN], auto step) {
+        if (LLMK_GEMM_ABL & 2) {                                  // the fragments count as used, nothing is multiplied
+#pragma unroll
+            for (int i = 0; i < TM; i++) asm volatile("" :: "v"(fa[i]));
+#pragma unroll
+            for (int j = 0; j < TN; j++) asm volatile("" :: "v"(fb[j]));
+            return;
+        }
 #pragma unroll
         for (int i = 0; i < TM; i++)
 #pragma unroll
@@ -409,6 +432,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     int par = 0;                        // stage s of the current work item lives in buffer (s + par) & 1
     issue(0, 0);
     if (nkb > 1) issue(1, 1);
+    abl_loads_on = false;
     bool st_young = false;              // the previous epilogue's stores are all issued and counted
 
     // Epilogues that read global memory (the pre-GELU activations, the old weight gradient) request it while the
@@ -602,7 +626,12 @@ gemm_pipelined_kernel(GemmArgs g) {
         // at chunk c ^ ((r >> 1) & 7). One 32-row block of the wave's tile goes through it at a time: every lane
         // writes the 4-column pieces it owns, then the wave reads the rows back 8 lanes to a row and stores
         // full 128-byte lines.
-        {
+        if (LLMK_GEMM_ABL & 8) {                                  // the accumulators count as used, nothing is stored
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) asm volatile("" :: "v"(acc[i][j]));
+        } else {
             char* strip = lds + STAGES * STAGE + wave * STRIP;
             const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
             constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
@@ -712,7 +741,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             }
         }
         if (!have_next) break;
-        st_young = cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
+        st_young = !(LLMK_GEMM_ABL & 8) && cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
         nkb = next_nkb;
     }
 #endif  // __HIP_DEVICE_COMPILE__

@@ -355,6 +355,58 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
     }
 }
 
+// Rows too wide for the register-resident kernel above (more than 8 vectors per lane: C > 4096 in bf16, > 2048 in fp32,
+// the GPT-3 descriptors of train_gpt2.cu:511-560 go to 12288): one 256-thread workgroup per row at a time, thread t owning
+// the vectors t, t + 256, ...; the row is read twice (sums, then the update; the second read comes from cache) and the
+// workgroup's dweight / dbias partials live in LDS (2 C floats) across all its rows. Same outputs and the same partial
+// layout as ln_backward_kernel, so the reduce kernel below serves both. Not tuned: no benchmarked model is this wide.
+__global__ void __launch_bounds__(256)
+ln_backward_wide_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const floatX* __restrict__ dout,
+                        const floatX* __restrict__ inp, const floatX* __restrict__ weight,
+                        const float* __restrict__ mean, const float* __restrict__ rstd, int N, int C) {
+    extern __shared__ float lds[];       // [2][C] partials, then 2 x 16 floats for the workgroup reductions
+    float* sdw = lds;
+    float* sdb = lds + C;
+    float* red = lds + 2 * (size_t)C;
+    const int nvec = C / VN;
+    const float invC = 1.0f / (float)C;
+    for (int c = threadIdx.x; c < 2 * C; c += 256) lds[c] = 0.f;
+    __syncthreads();
+    for (int row = blockIdx.x; row < N; row += gridDim.x) {
+        const size_t base = (size_t)row * C;
+        const float m = mean[row], r = rstd[row];
+        float a = 0.f, bsum = 0.f;
+        for (int v = threadIdx.x; v < nvec; v += 256) {
+            const vecX g = ld_vec(dout + base + (size_t)v * VN), x = ld_vec(inp + base + (size_t)v * VN), w = ld_vec(weight + (size_t)v * VN);
+#pragma unroll
+            for (int k = 0; k < VN; k++) {
+                const float nh = (to_f32(x[k]) - m) * r, dn = to_f32(w[k]) * to_f32(g[k]);
+                a += dn;
+                bsum += dn * nh;
+            }
+        }
+        a = block_reduce<false>(a, red) * invC;
+        bsum = block_reduce<false>(bsum, red + 16) * invC;
+        for (int v = threadIdx.x; v < nvec; v += 256) {
+            const vecX g = ld_vec(dout + base + (size_t)v * VN), x = ld_vec(inp + base + (size_t)v * VN), w = ld_vec(weight + (size_t)v * VN);
+            const vecX di = ld_vec(dinp + base + (size_t)v * VN);
+            vecX o;
+#pragma unroll
+            for (int k = 0; k < VN; k++) {
+                const float gk = to_f32(g[k]);
+                const float nh = (to_f32(x[k]) - m) * r, dn = to_f32(w[k]) * gk;
+                sdb[v * VN + k] += gk;                        // column v * VN + k belongs to this thread alone
+                sdw[v * VN + k] += nh * gk;
+                o[k] = from_f32<floatX>(to_f32(di[k]) + (dn - a - nh * bsum) * r);
+            }
+            st_vec(dinp + base + (size_t)v * VN, o);
+        }
+        __syncthreads();                                      // the reduction slots are reused by the next row
+    }
+    float* out = partial + (size_t)blockIdx.x * 2 * C;
+    for (int c = threadIdx.x; c < 2 * C; c += 256) out[c] = lds[c];
+}
+
 // dweight[c] += sum_blocks partial[b][0][c]; dbias likewise. A workgroup owns 32 columns; its 32 row
 // groups each add every 32nd partial in ascending order, then the 32 sub-sums are added in group order:
 // a fixed summation tree, so the result is reproducible, with 32x the memory parallelism of one thread
@@ -424,10 +476,29 @@ void llmk_layernorm_backward(void* dinp, void* dweight, void* dbias, float* scra
     if (llmk::failed()) return;
     LLMK_REQUIRE(C > 0 && C % VN == 0, "layernorm_backward: C=%d must be a multiple of %d", C, VN);
     const int nv = CEIL_DIV(C / VN, 64);
-    LLMK_REQUIRE(nv <= 8, "layernorm_backward: C=%d too large (max %d)", C, 8 * 64 * VN);
     const int N = B * T;
     if (N == 0) return;
     hipStream_t st = (hipStream_t)stream;
+    if (nv > 8) {                                             // wider than the register-resident kernel takes
+        const size_t smem = (2 * (size_t)C + 32) * sizeof(float);
+        LLMK_REQUIRE(smem <= 160 * 1024, "layernorm_backward: C=%d too large (max %d)", C, (160 * 1024 / 4 - 32) / 2);
+        const int blocks = min(ln_backward_blocks(), N);
+        {
+            llmk::ProfScope prof("layernorm_backward", 0, 4.0 * N * C * sizeof(floatX) + 2.0 * N * sizeof(float), st);
+            static bool attr_set = false;
+            if (!attr_set) {
+                HIP_CHECK(hipFuncSetAttribute((const void*)ln_backward_wide_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+                attr_set = true;
+            }
+            ln_backward_wide_kernel<<<blocks, 256, smem, st>>>((floatX*)dinp, scratch, (const floatX*)dout, (const floatX*)inp,
+                                                             (const floatX*)weight, mean, rstd, N, C);
+            LAUNCH_CHECK();
+        }
+        llmk::ProfScope prof2("layernorm_backward_reduce", 0, (double)blocks * 2 * C * sizeof(float), st);
+        ln_backward_reduce_kernel<<<CEIL_DIV(2 * C, LNR_COLS), LNR_COLS * LNR_GROUPS, 0, st>>>((floatX*)dweight, (floatX*)dbias, scratch, blocks, C);
+        LAUNCH_CHECK();
+        return;
+    }
     const int waves = lnb_waves(nv);
     const int blocks = min(ln_backward_blocks(), CEIL_DIV(N, waves));
     const size_t smem = (size_t)(waves - 1) * 2 * C * sizeof(float);

@@ -7,7 +7,7 @@ events on the launch stream (llmk_profile_*), so a case that launches several ke
 dweight GEMM, split-K reduce, bias gradient) reports each of them. Inputs are N(0,1) from a fixed seed, weights
 N(0,0.02). Before each repetition 1 GiB is overwritten, which evicts the 8 x 4 MiB L2s and the 256 MiB Infinity Cache.
 
-    python llm.c_amd/microbench.py [--reps 20] [--only gemm,attention,...] [--json out.json]
+    python llm.c_amd/microbench.py [--reps 20] [--only gemm,attention,...] [--json out.json] [--variant NAME]
 
 Prints, per kernel family and case: median and minimum milliseconds, the algorithmic TFLOP/s or GB/s at the median,
 and the fraction of the roofline that bounds the family (2500 TFLOP/s bf16 MFMA, 8000 GB/s HBM). PyTorch is used
@@ -196,7 +196,11 @@ def main():
     ap.add_argument("--reps", type=int, default=20)
     ap.add_argument("--only", default="")
     ap.add_argument("--json", default="")
+    ap.add_argument("--variant", default="", help="time lib/variants/NAME/libllmk_bf16.so (python llm.c_amd/build.py --variant NAME "
+                    "-D...: a build with ablation switches set, whose results are wrong by design) instead of the product library")
     args = ap.parse_args()
+    if args.variant:
+        pkg.LIBDIR = os.path.join(pkg.LIBDIR, "variants", args.variant)
     L = pkg.load("bf16")          # raises LibraryMissing when the HIP library has not been built
     L.llmk_init(0)
     results = run_cases(L, args.reps, [s for s in args.only.split(",") if s], lambda line: print(line, flush=True))

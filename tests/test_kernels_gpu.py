@@ -132,10 +132,9 @@ def test_layernorm_forward_and_fused_residual(precision, N, C):
 
 
 @pytest.mark.parametrize("precision", PRECS)
-@pytest.mark.parametrize("N,C", [(9, 64), (2048, 768), (520, 1600), (300, 1024), (45, 2048), (70, 2560), (37, 4096)])
+@pytest.mark.parametrize("N,C", [(9, 64), (2048, 768), (520, 1600), (300, 1024), (45, 2048), (70, 2560), (37, 4096),
+                                 (300, 5120), (19, 12288)])      # past 8 vectors per lane: the workgroup-per-row kernel
 def test_layernorm_backward(precision, N, C):
-    if precision == "fp32" and C > 2048:
-        pytest.skip("the fp32 kernel holds a row in at most 8 vectors of 4 per lane: C <= 2048")
     L = G.lib(precision)
     x, g = G.rounded(rnd((N, C), 0, 1.5), precision), G.rounded(rnd((N, C), 1), precision)
     w = G.rounded(rnd(C, 2), precision)
