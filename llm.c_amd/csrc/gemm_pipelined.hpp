@@ -443,10 +443,32 @@ gemm_pipelined_kernel(GemmArgs g) {
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
     // GELU backward: the pre-activation values of the 16 bytes each lane stores per (block, pass, quarter), as it stores them
     u32x4 pre_act[epi_gelu_bwd(EPI) ? TM : 1][epi_gelu_bwd(EPI) ? PASSES : 1][4];
+    // Row groups of a tile that lies wholly inside the output (no lane tests its row or column): 8 rows x 128 B, lane
+    // (row = lane / 8, chunk = lane % 8) at a wave-uniform base (scalar registers) plus one per-lane byte offset that is the
+    // same for every group of every tile. The general form costs each load and store a 64-bit address of its own.
+    const unsigned row_lane_off = (unsigned)(((lane >> 3) * g.ldc + (lane & 7) * 8) * (int)sizeof(floatX));
+    auto group_ptr = [&](const floatX* buf, int row0, int col0) -> char* {
+        const size_t off = ((size_t)row0 * g.ldc + col0) * sizeof(floatX);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)off);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(off >> 32));
+        return const_cast<char*>(reinterpret_cast<const char*>(buf)) + (((size_t)hi << 32) | lo) + row_lane_off;
+    };
+    // (measured: 4 % off the kernel whose epilogue only multiplies by a stored derivative, which is short of registers and
+    // of little else; 1-2 % slower for the epilogues with activation math, so only that one takes this form)
+    constexpr bool UNIFORM_GROUPS = EPI == EPI_DGELU_D;
+    bool tile_inside = false;            // the tile whose epilogue is running (or about to) lies wholly inside the output
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
         if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
         if constexpr (epi_gelu_bwd(EPI)) {
+            if (tile_inside) {
+#pragma unroll
+                for (int pass = 0; pass < PASSES; pass++)
+#pragma unroll
+                    for (int t = 0; t < 4; t++)
+                        pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(group_ptr(g.aux, wm0 + i * 32 + t * 8, wn0 + pass * 64));
+                return;
+            }
 #pragma unroll
             for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
@@ -572,6 +594,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         {
             const unsigned cur = buf_of(nst - 1);
             request_bias(n0);                                     // nothing of this wave is in flight here (kernels with a bias)
+            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
             prefetch_epilogue(m0, n0, 0);
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
@@ -700,15 +723,23 @@ gemm_pipelined_kernel(GemmArgs g) {
                             }
                         } else {
                             const int n = wn0 + pass * 64 + ch * 8;
-                            if (m < g.M && n < g.N) {
-                                const size_t o = (size_t)m * g.ldc + n;
+                            if (tile_inside || (m < g.M && n < g.N)) {
+                                u32x4 *cptr, *auxptr = nullptr;
+                                if (tile_inside) {
+                                    cptr = reinterpret_cast<u32x4*>(group_ptr(g.C, wm0 + i * 32 + t * 8, wn0 + pass * 64));
+                                    if (epi_gelu_fwd(EPI)) auxptr = reinterpret_cast<u32x4*>(group_ptr(g.aux, wm0 + i * 32 + t * 8, wn0 + pass * 64));
+                                } else {
+                                    const size_t o = (size_t)m * g.ldc + n;
+                                    cptr = reinterpret_cast<u32x4*>(g.C + o);
+                                    if (epi_gelu_fwd(EPI)) auxptr = reinterpret_cast<u32x4*>(g.aux + o);
+                                }
                                 union { u32x4 u; bf16x8 h; } x, y;
                                 x.u = raw;
                                 if (EPI == EPI_BIAS_GELU) {
-                                    st_out(reinterpret_cast<u32x4*>(g.aux + o), x.u);
+                                    st_out(auxptr, x.u);
 #pragma unroll
                                     for (int e = 0; e < 8; e++) y.h[e] = (__bf16)gelu_f((float)x.h[e]);
-                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                    st_out(cptr, y.u);
                                 } else if (EPI == EPI_BIAS_GELU_D) {
                                     union { u32x4 u; bf16x8 h; } d;
 #pragma unroll
@@ -717,8 +748,8 @@ gemm_pipelined_kernel(GemmArgs g) {
                                         y.h[e] = (__bf16)gelu_with_grad_f((float)x.h[e], gr);
                                         d.h[e] = (__bf16)gr;
                                     }
-                                    st_out(reinterpret_cast<u32x4*>(g.aux + o), d.u);
-                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                    st_out(auxptr, d.u);
+                                    st_out(cptr, y.u);
                                 } else if (epi_gelu_bwd(EPI)) {
                                     // the product of the rounded gradient and gelu'(pre), as gelu_backward_inplace forms it
                                     // (EPI_DGELU_D: gelu'(pre) is what was stored)
@@ -727,9 +758,9 @@ gemm_pipelined_kernel(GemmArgs g) {
 #pragma unroll
                                     for (int e = 0; e < 8; e++)
                                         y.h[e] = (__bf16)((EPI == EPI_DGELU_D ? (float)pa.h[e] : gelu_grad_f((float)pa.h[e])) * (float)x.h[e]);
-                                    st_out(reinterpret_cast<u32x4*>(g.C + o), y.u);
+                                    st_out(cptr, y.u);
                                 } else {
-                                    st_out(reinterpret_cast<u32x4*>(g.C + o), x.u);
+                                    st_out(cptr, x.u);
                                 }
                             }
                         }
