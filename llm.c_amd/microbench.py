@@ -95,6 +95,9 @@ def run_cases(L, reps=20, only=(), emit=print):
                 pre = torch.empty_like(out_t)
                 report(f"matmul_forward+gelu {nm} K={K} OC={OC}",
                        measure(lambda: L.llmk_matmul_forward(p(out_t), p(inp), p(w), p(bias), B, T, K, OC, None, p(pre), 2)))
+                # gelu_fusion 3: the second output is gelu'(pre-activation), kept for the backward epilogue
+                report(f"matmul_forward+gelu3 {nm} K={K} OC={OC}",
+                       measure(lambda: L.llmk_matmul_forward(p(out_t), p(inp), p(w), p(bias), B, T, K, OC, None, p(pre), 3)))
                 del pre
             dout = out_t.normal_(generator=g)                  # reuse the output buffer as the upstream gradient
             dinp, dw = torch.empty_like(inp), torch.zeros_like(w)
@@ -106,6 +109,8 @@ def run_cases(L, reps=20, only=(), emit=print):
                 pre = randn(N, K)
                 report(f"matmul_backward+dgelu {nm} K={K} OC={OC}",
                        measure(lambda: L.llmk_matmul_backward(p(dinp), p(dw), p(dbias), p(dout), p(inp), p(w), p(scratch), B, T, K, OC, None, p(pre), 2)))
+                report(f"matmul_backward+dgelu3 {nm} K={K} OC={OC}",      # pre holds a stored derivative here (any values do for timing)
+                       measure(lambda: L.llmk_matmul_backward(p(dinp), p(dw), p(dbias), p(dout), p(inp), p(w), p(scratch), B, T, K, OC, None, p(pre), 3)))
                 del pre
             del inp, w, out_t, dout, dinp, dw, scratch
             torch.cuda.empty_cache()
