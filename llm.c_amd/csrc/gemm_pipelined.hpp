@@ -31,6 +31,7 @@
 #include "common.hpp"
 #include "gelu.hpp"
 #include <type_traits>
+#include <utility>
 
 namespace gemmk {
 
@@ -86,6 +87,15 @@ constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 #ifndef LLMK_GEMM_ABL
 #define LLMK_GEMM_ABL 0
 #endif
+// Switch for a measured alternative, off in the product: the last K stage of a tile taken one 32-row block at a time, each
+// finished block's epilogue (strip pass and stores) placed behind the matrix instructions of the next block, the barrier and
+// the tile change before the last block. Bit-exact; it needs 20 more registers (253-255) and, timed against the product on
+// one machine, alternating: NT bias kernels +2 to +5 % (fc 0.340 -> 0.347 ms, fcproj 0.275 -> 0.290, qkv 0.210 -> 0.219), NT
+// GELU +1 to +3 %, NN store within +-1 %. python llm.c_amd/build.py --variant rowwise -DLLMK_ROWWISE_LAST=1 builds it for
+// llm.c_amd/microbench.py --variant rowwise (2: also the GELU-backward kernels).
+#ifndef LLMK_ROWWISE_LAST
+#define LLMK_ROWWISE_LAST 0
+#endif
 constexpr int PBK = 64;                 // K per stage
 constexpr int STAGES = 2;               // operand buffers: one being multiplied, one being filled
 constexpr int KGRAN = PBK;              // K (and the K range of a split) must be a multiple of this
@@ -95,6 +105,12 @@ constexpr int LDS_TOTAL = 160 * 1024;
 constexpr int smem_bytes(int bm, int bn, int nw) { return STAGES * (bm + bn) * PBK * 2 + nw * 32 * 128; }
 
 typedef __attribute__((address_space(3))) void* lds_void_ptr;
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): loops whose index has to be a constant expression
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F& f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>{}), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>{}); }
 
 // wait until at most N of this wave's vector-memory operations are outstanding (gfx9 encoding, other counters untouched)
 template <int N>
@@ -527,140 +543,21 @@ gemm_pipelined_kernel(GemmArgs g) {
         }
     };
 
-    while (true) {
-        const int m0 = tile_m * BM, n0 = tile_n * BN;
-#pragma unroll
-        for (int i = 0; i < TM; i++)
-#pragma unroll
-            for (int j = 0; j < TN; j++)
-#pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
-        if constexpr (ROWSUM) {
-            rowsum_step = tile_n == 0 ? wn : -1;
-#pragma unroll
-            for (int i = 0; i < TM; i++) rsum[i] = 0.f;
-        }
-
-        // ---- K loop over stages of 64, software-pipelined: the operands of the next 16-wide step (and the
-        // barrier that publishes the next stage) are requested while the matrix cores work on the current step.
-        // Stage s lives in buffer (s + par) & 1; while it is multiplied, stage s+1 is in flight.
-        bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
-        const int nst = nkb;
-        // the next work item's coordinates are worked out here (integer divisions), under the K loop's MFMAs
-        int next_m, next_n, next_split, next_kbeg = 0, next_nkb = 0;
-        const bool have_next = work_item(it + 1, next_m, next_n, next_split, next_kbeg, next_nkb);
-        auto buf_idx = [&](int st) -> int { return (st + par) & 1; };
-        auto buf_of = [&](int st) -> unsigned { return (unsigned)buf_idx(st) * STAGE; };
-        // The last-but-one stage frees a buffer a whole stage before the tile ends: the next work item's first stage
-        // is requested into it there and then instead of at the tile change, and the next item's stages alternate
-        // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
-        // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
-        // short of scalar registers).
-        constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
-        bool early0 = false;
-        if (have_next) {
-            if constexpr (EARLY0) {
-                early0 = nst >= 2 && !voff_edge && !is_edge(next_m, next_n);
-                if (early0) bases_into(tile_base_n, next_m * BM, next_n * BN, next_kbeg);
-            }
-        }
-        if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
-        else wait_vmcnt<0>();
-        barrier_no_fence();                                       // stage 0 landed for everyone
-        read_frags(buf_of(0), S0{}, fa0, fb0);
-        for (int st = 0; st < nst - 1; st++) {
-            const unsigned cur = buf_of(st);
-            read_frags(cur, S1{}, fa1, fb1);
-            await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0, S0{});
-            if (late && st >= 1) issue(st + 1, buf_idx(st + 1));
-            read_frags(cur, S2{}, fa0, fb0);
-            await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1, S1{});
-            read_frags(cur, S3{}, fa1, fb1);
-            await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0, S2{});
-            __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
-            if (st == 0 && st_young) wait_vmcnt<NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
-            barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
-            if (!late) {
-                if (st + 2 < nst) issue(st + 2, buf_idx(st));
-                else if (EARLY0 && !HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(st));
-            }
-            read_frags(buf_of(st + 1), S0{}, fa0, fb0);
-            await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1, S3{});
-        }
+    // ---- epilogue of one 32-row block of this wave's tile ---------------------------------------------
+    // Wave-private staging strip behind the operand buffers: 32 rows x 128 B, the 16-byte chunk c of row r stored
+    // at chunk c ^ ((r >> 1) & 7). One 32-row block of the wave's tile goes through it at a time: every lane
+    // writes the 4-column pieces it owns, then the wave reads the rows back 8 lanes to a row and stores
+    // full 128-byte lines. e_m0, e_n0, e_split: the tile (they outlive the tile change, which renames the current one).
+    int e_m0 = 0, e_n0 = 0, e_split = 0;
+    auto epi_block = [&](auto ic) {
+        constexpr int i = decltype(ic)::value;
+        const int cur_m0 = e_m0, cur_n0 = e_n0, cur_split = e_split;
+        char* strip = lds + STAGES * STAGE + wave * STRIP;
+        const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
+        constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
+        const int wswz = (idx >> 1) & 7;
+        (void)cur_split;
         {
-            const unsigned cur = buf_of(nst - 1);
-            request_bias(n0);                                     // nothing of this wave is in flight here (kernels with a bias)
-            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
-            prefetch_epilogue(m0, n0, 0);
-            read_frags(cur, S1{}, fa1, fb1);
-            await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0, S0{});
-            if (EARLY0 && !HAS_BIAS && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
-            read_frags(cur, S2{}, fa0, fb0);
-            await_frags(fa1, fb1, Younger{});
-            mma(fa1, fb1, S1{});
-            bias_ready();                                         // two 16-wide steps after the request
-            if (EARLY0 && HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
-            read_frags(cur, S3{}, fa1, fb1);
-            await_frags(fa0, fb0, Younger{});
-            mma(fa0, fb0, S2{});
-            await_frags(fa1, fb1, NoneYounger{});
-            mma(fa1, fb1, S3{});
-        }
-
-        // ---- request the next work item's first K blocks, then run the epilogue under them --------
-        barrier_no_fence();                                  // every wave is done reading both buffers
-        const int cur_m0 = m0, cur_n0 = n0, cur_split = split;
-        if constexpr (ROWSUM) {
-            if (rowsum_step >= 0) {                               // the two k halves of a row sit 32 lanes apart
-#pragma unroll
-                for (int i = 0; i < TM; i++) {
-                    const float s = rsum[i] + __shfl_xor(rsum[i], 32, 64);
-                    const int m = cur_m0 + wm * WTM + i * 32 + idx;
-                    if (half == 0 && m < g.M) g.rowsum[((size_t)cur_split * WGN + wn) * g.M + m] = s;
-                }
-            }
-        }
-        prefetch_epilogue(cur_m0, cur_n0, 1);                     // before the next tile's loads: it is needed before them
-        it++;
-        if (have_next) {
-            tile_m = next_m; tile_n = next_n; split = next_split;
-            kbeg = next_kbeg;
-            if (EARLY0 && early0) {                               // its first stage is already on the way, in the buffer of stage nst-2
-                tile_base[0] = tile_base_n[0]; tile_base[1] = tile_base_n[1];
-                par = (nst - 2 + par) & 1;
-            } else {
-                setup_bases(tile_m * BM, tile_n * BN, kbeg);
-                const bool edge = is_edge(tile_m, tile_n);
-                if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
-                voff_edge = edge;
-                par = 0;
-                issue(0, 0);
-            }
-            if (next_nkb > 1) issue(1, (1 + par) & 1);
-        }
-
-        // ---- epilogue ---------------------------------------------------------------------------------
-        // Wave-private staging strip behind the operand buffers: 32 rows x 128 B, the 16-byte chunk c of row r stored
-        // at chunk c ^ ((r >> 1) & 7). One 32-row block of the wave's tile goes through it at a time: every lane
-        // writes the 4-column pieces it owns, then the wave reads the rows back 8 lanes to a row and stores
-        // full 128-byte lines.
-        if (LLMK_GEMM_ABL & 8) {                                  // the accumulators count as used, nothing is stored
-#pragma unroll
-            for (int i = 0; i < TM; i++)
-#pragma unroll
-                for (int j = 0; j < TN; j++) asm volatile("" :: "v"(acc[i][j]));
-        } else {
-            char* strip = lds + STAGES * STAGE + wave * STRIP;
-            const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
-            constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
-            const int wswz = (idx >> 1) & 7;
-#pragma unroll
-            for (int i = 0; i < TM; i++) {
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++) {
                     // phase 1: lane (row = idx, half) owns columns 8q + 4*half + 0..3 of each 32-column block
@@ -769,10 +666,209 @@ gemm_pipelined_kernel(GemmArgs g) {
                     __builtin_amdgcn_wave_barrier();
                 }
                 prefetch_epilogue(cur_m0, cur_n0, i + 2);
+        }
+    };
+
+    while (true) {
+        const int m0 = tile_m * BM, n0 = tile_n * BN;
+#pragma unroll
+        for (int i = 0; i < TM; i++)
+#pragma unroll
+            for (int j = 0; j < TN; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+        if constexpr (ROWSUM) {
+            rowsum_step = tile_n == 0 ? wn : -1;
+#pragma unroll
+            for (int i = 0; i < TM; i++) rsum[i] = 0.f;
+        }
+
+        // ---- K loop over stages of 64, software-pipelined: the operands of the next 16-wide step (and the
+        // barrier that publishes the next stage) are requested while the matrix cores work on the current step.
+        // Stage s lives in buffer (s + par) & 1; while it is multiplied, stage s+1 is in flight.
+        bf16x8 fa0[TM], fb0[TN], fa1[TM], fb1[TN];
+        const int nst = nkb;
+        // the next work item's coordinates are worked out here (integer divisions), under the K loop's MFMAs
+        int next_m, next_n, next_split, next_kbeg = 0, next_nkb = 0;
+        const bool have_next = work_item(it + 1, next_m, next_n, next_split, next_kbeg, next_nkb);
+        auto buf_idx = [&](int st) -> int { return (st + par) & 1; };
+        auto buf_of = [&](int st) -> unsigned { return (unsigned)buf_idx(st) * STAGE; };
+        // The last-but-one stage frees a buffer a whole stage before the tile ends: the next work item's first stage
+        // is requested into it there and then instead of at the tile change, and the next item's stages alternate
+        // from that buffer on (interior tiles only: they share the lane offsets; not with the += epilogue, whose reads of the old
+        // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
+        // short of scalar registers).
+        constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
+        constexpr bool ROWWISE = LLMK_ROWWISE_LAST && EARLY0 && !TR_ASM && (!epi_gelu_bwd(EPI) || LLMK_ROWWISE_LAST >= 2);
+        bool early0 = false;
+        if (have_next) {
+            if constexpr (EARLY0) {
+                early0 = nst >= 2 && !voff_edge && !is_edge(next_m, next_n);
+                if (early0) bases_into(tile_base_n, next_m * BM, next_n * BN, next_kbeg);
+            }
+        }
+        // (with the row-wise last stage a tile's stores are only counted as younger when its successor's first stage was
+        // requested ahead of them, half of them ahead of its second stage)
+        if (nst >= 2) { if (st_young) wait_vmcnt<CPW + NS_EPI>(); else wait_vmcnt<CPW>(); }
+        else wait_vmcnt<0>();
+        barrier_no_fence();                                       // stage 0 landed for everyone
+        read_frags(buf_of(0), S0{}, fa0, fb0);
+        for (int st = 0; st < nst - 1; st++) {
+            const unsigned cur = buf_of(st);
+            read_frags(cur, S1{}, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0, S0{});
+            if (late && st >= 1) issue(st + 1, buf_idx(st + 1));
+            read_frags(cur, S2{}, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1, S1{});
+            read_frags(cur, S3{}, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0, S2{});
+            __builtin_amdgcn_s_waitcnt(0xC07F);                   // lgkmcnt(0): this wave is done reading stage st
+            if (st == 0 && st_young) wait_vmcnt<ROWWISE ? NS_EPI / 2 : NS_EPI>(); else wait_vmcnt<0>();     // stage st+1 has landed (this wave's share)
+            barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
+            if (!late) {
+                if (st + 2 < nst) issue(st + 2, buf_idx(st));
+                else if (EARLY0 && !HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(st));
+            }
+            read_frags(buf_of(st + 1), S0{}, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1, S3{});
+        }
+        // what happens between the last read of this tile's operands and the epilogue's end: the next work item becomes the
+        // current one and its first stages are requested
+        auto tile_change = [&]() {
+            it++;
+            if (!have_next) return;
+            tile_m = next_m; tile_n = next_n; split = next_split;
+            kbeg = next_kbeg;
+            if (EARLY0 && early0) {                               // its first stage is already on the way, in the buffer of stage nst-2
+                tile_base[0] = tile_base_n[0]; tile_base[1] = tile_base_n[1];
+                par = (nst - 2 + par) & 1;
+            } else {
+                setup_bases(tile_m * BM, tile_n * BN, kbeg);
+                const bool edge = is_edge(tile_m, tile_n);
+                if (edge || voff_edge) setup_voff(tile_m * BM, tile_n * BN);
+                voff_edge = edge;
+                par = 0;
+                issue(0, 0);
+            }
+            if (next_nkb > 1) issue(1, (1 + par) & 1);
+        };
+        e_m0 = m0; e_n0 = n0; e_split = split;
+        if constexpr (ROWWISE) {
+            // The last stage by 32-row blocks: the B fragments of all four steps are held, block i takes its A fragments and
+            // its 4 x TN matrix instructions, and the finished block i - 1 goes through the strip and out behind them. The
+            // operands are read for the last time before the final block's matrix instructions: the barrier and the tile
+            // change sit there, two blocks of output stores ahead of the next tile's second stage and two behind it.
+            const unsigned cur = buf_of(nst - 1);
+            request_bias(n0);
+            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
+            prefetch_epilogue(m0, n0, 0);
+            prefetch_epilogue(m0, n0, 1);
+            bf16x8 fbs[3][TN], far[2][3];
+            auto read_b = [&](auto sc, bf16x8 (&fb)[TN]) {
+                constexpr int S = decltype(sc)::value;
+#pragma unroll
+                for (int j = 0; j < TN; j++) {
+                    if (LLMK_GEMM_ABL & 4) asm volatile("" : "+v"(fb[j]));
+                    else if constexpr (B_T) fb[j] = frag_t(bbase[j] + cur, std::integral_constant<int, S * 16 * BN * 2>{}, std::integral_constant<int, (S * 16 + 4) * BN * 2>{});
+                    else fb[j] = frag_k(bbase[j] + cur, S);
+                }
+            };
+            auto read_a = [&](auto ic, bf16x8 (&fa)[3]) {
+                constexpr int i = decltype(ic)::value;
+                static_for<3>([&](auto sc) {
+                    constexpr int S = decltype(sc)::value + 1;
+                    if (LLMK_GEMM_ABL & 4) asm volatile("" : "+v"(fa[S - 1]));
+                    else fa[S - 1] = frag_k(abase[i] + cur, S);
+                });
+            };
+            static_assert(!A_T, "row-wise last stage: A fragments are K-contiguous");
+            auto mfma1 = [&](f32x16& c, const bf16x8& b, const bf16x8& a) {
+                if (LLMK_GEMM_ABL & 2) asm volatile("" :: "v"(a), "v"(b));
+                else c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(b, a, c, 0, 0, 0);
+            };
+            read_b(S1{}, fbs[0]);
+            read_a(std::integral_constant<int, 0>{}, far[0]);
+            read_b(S2{}, fbs[1]);
+            read_b(S3{}, fbs[2]);
+            static_for<TM>([&](auto ic) {
+                constexpr int i = decltype(ic)::value;
+                if constexpr (i + 1 < TM) read_a(std::integral_constant<int, i + 1>{}, far[(i + 1) & 1]);
+                if constexpr (i == TM - 1) {
+                    __builtin_amdgcn_s_waitcnt(0xC07F);           // lgkmcnt(0): this wave is done reading the operand buffers
+                    barrier_no_fence();                           // ... and so is everyone
+                    tile_change();
+                }
+#pragma unroll
+                for (int j = 0; j < TN; j++) mfma1(acc[i][j], fb0[j], fa0[i]);
+#pragma unroll
+                for (int sidx = 0; sidx < 3; sidx++)
+#pragma unroll
+                    for (int j = 0; j < TN; j++) mfma1(acc[i][j], fbs[sidx][j], far[i & 1][sidx]);
+                if constexpr (i == 0) {
+                    bias_ready();
+                    if (early0 && (HAS_BIAS || late)) issue_from(tile_base_n, 0, buf_idx(nst - 2));   // (the early waves of a kernel without bias: one stage ago)
+                }
+                if constexpr (i >= 1) {
+                    if (!(LLMK_GEMM_ABL & 8)) epi_block(std::integral_constant<int, i - 1>{});
+                }
+            });
+        } else {
+            const unsigned cur = buf_of(nst - 1);
+            request_bias(n0);                                     // nothing of this wave is in flight here (kernels with a bias)
+            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
+            prefetch_epilogue(m0, n0, 0);
+            read_frags(cur, S1{}, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0, S0{});
+            if (EARLY0 && !HAS_BIAS && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
+            read_frags(cur, S2{}, fa0, fb0);
+            await_frags(fa1, fb1, Younger{});
+            mma(fa1, fb1, S1{});
+            bias_ready();                                         // two 16-wide steps after the request
+            if (EARLY0 && HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
+            read_frags(cur, S3{}, fa1, fb1);
+            await_frags(fa0, fb0, Younger{});
+            mma(fa0, fb0, S2{});
+            await_frags(fa1, fb1, NoneYounger{});
+            mma(fa1, fb1, S3{});
+
+            // ---- request the next work item's first K blocks, then run the epilogue under them --------
+            barrier_no_fence();                                  // every wave is done reading both buffers
+            if constexpr (ROWSUM) {
+                if (rowsum_step >= 0) {                               // the two k halves of a row sit 32 lanes apart
+#pragma unroll
+                    for (int i = 0; i < TM; i++) {
+                        const float s = rsum[i] + __shfl_xor(rsum[i], 32, 64);
+                        const int m = e_m0 + wm * WTM + i * 32 + idx;
+                        if (half == 0 && m < g.M) g.rowsum[((size_t)e_split * WGN + wn) * g.M + m] = s;
+                    }
+                }
+            }
+            prefetch_epilogue(e_m0, e_n0, 1);                     // before the next tile's loads: it is needed before them
+            tile_change();
+        }
+        const int cur_m0 = e_m0, cur_n0 = e_n0;
+
+        // ---- epilogue (what the last stage did not already take) ---------------------------------------
+        if (LLMK_GEMM_ABL & 8) {                                  // the accumulators count as used, nothing is stored
+#pragma unroll
+            for (int i = 0; i < TM; i++)
+#pragma unroll
+                for (int j = 0; j < TN; j++) asm volatile("" :: "v"(acc[i][j]));
+        } else {
+            if constexpr (ROWWISE) {
+                epi_block(std::integral_constant<int, TM - 1>{});
+            } else {
+                static_for<TM>([&](auto ic) { epi_block(ic); });
             }
         }
         if (!have_next) break;
-        st_young = !(LLMK_GEMM_ABL & 8) && cur_m0 + BM <= g.M && cur_n0 + BN <= g.N;    // interior tile: every lane stored, NS_EPI stores per wave
+        st_young = !(LLMK_GEMM_ABL & 8) && cur_m0 + BM <= g.M && cur_n0 + BN <= g.N     // interior tile: every lane stored, NS_EPI stores per wave
+                   && (!ROWWISE || early0);
         nkb = next_nkb;
     }
 #endif  // __HIP_DEVICE_COMPILE__
