@@ -629,7 +629,7 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
     auto load_stats = [&](int qi) {
         const int q = 64 * qi + (tid & 63);
         if (tid < 64) rstat = q < T ? lbase[q] * LOG2E : 0.f;
-        else if (tid < 128) rstat = q < T ? dbase[q] : 0.f;
+        else if (tid < 128) rstat = q < T ? -dbase[q] : 0.f;          // negated: it is the start value of the dP accumulator
     };
     auto store_stats = [&](int buf) {
         if (tid < 64) sL[buf][tid] = rstat;
@@ -659,20 +659,27 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
         for (int qb = 0; qb < 2; qb++) {
             const int q0 = 64 * qi + 32 * qb;
             if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
+            // dP - rowsum(dO*O) comes out of the matrix cores: the accumulator of dO.V^T starts from -rowsum(dO*O) of its
+            // 16 queries (an accumulator register is a query here), which takes a subtraction per score off the vector ALU
             f32x16 sacc, pacc;
 #pragma unroll
-            for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+            for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
-            for (int s = 0; s < 4; s++) {
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
-                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s, lane), vf[s], pacc, 0, 0, 0);
+            for (int g = 0; g < 4; g++) {
+                const f32x4 d4 = *reinterpret_cast<const f32x4*>(&sD[buf][32 * qb + g * 8 + half * 4]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) pacc[4 * g + e] = d4[e];
             }
-            f32x4 d4[4];
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
+#pragma unroll
+            for (int s = 0; s < 4; s++)
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s, lane), vf[s], pacc, 0, 0, 0);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int rr = 32 * qb + g * 8 + half * 4;
                 const f32x4 l4 = *reinterpret_cast<const f32x4*>(&sL[buf][rr]);
-                d4[g] = *reinterpret_cast<const f32x4*>(&sD[buf][rr]);
 #pragma unroll
                 for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
             }
@@ -684,17 +691,20 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
                 }
             }
 #pragma unroll
-            for (int g = 0; g < 4; g++)
-#pragma unroll
-                for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[g][e]);
+            for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * pacc[r];
 #pragma unroll
             for (int s2 = 0; s2 < 2; s2++) {
-                const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
+                const bf16x8 pf = pack_acc(sacc, s2);
 #pragma unroll
-                for (int d = 0; d < 2; d++) {
+                for (int d = 0; d < 2; d++)
                     dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tdo, 32 * qb + 16 * s2, 32 * d, lane), pf, dv[d], 0, 0, 0);
+            }
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                const bf16x8 dsf = pack_acc(pacc, s2);
+#pragma unroll
+                for (int d = 0; d < 2; d++)
                     dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_cols_accorder(tq, 32 * qb + 16 * s2, 32 * d, lane), dsf, dk[d], 0, 0, 0);
-                }
             }
         }
         if (more) {
@@ -725,7 +735,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                         const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH, int nk) {
     __shared__ __attribute__((aligned(1024))) char sQ[2][SW_TILE];
     __shared__ __attribute__((aligned(1024))) char sdO[2][SW_TILE];
-    extern __shared__ __attribute__((aligned(16))) float sStat[];   // [2][T]: log-sum-exp (in log2 units) and rowsum(dO*O) of every query of this head
+    extern __shared__ __attribute__((aligned(16))) float sStat[];   // [2][T]: log-sum-exp (in log2 units) and -rowsum(dO*O) of every query of this head
     float* sLall = sStat;
     float* sDall = sStat + T;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, idx = lane & 31, half = lane >> 5;
@@ -760,7 +770,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
         }
         // the per-query statistics of the head go to LDS once (the first tile's queries include the second's): no global
         // loads besides the tiles inside the loops
-        for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = dbase[q]; }
+        for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = -dbase[q]; }    // negated: see below
     }
     int buf = 0;
 
@@ -806,14 +816,25 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
             for (int qb = 0; qb < 2; qb++) {
                 const int q0 = 64 * qi + 32 * qb;
                 if (q0 + 31 < kw0) continue;                 // all 32 queries precede every key of this wave
+                // the accumulator of dO.V^T starts from -rowsum(dO*O) of its 16 queries (see fa_backward_dkdv_kernel)
                 f32x16 sacc, pacc;
 #pragma unroll
-                for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
+                for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
-                for (int s = 0; s < 4; s++) {
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
-                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
+                for (int g = 0; g < 4; g++) {
+                    const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) pacc[4 * g + e] = d4[e];
                 }
+                // one chain after the other, S first: its exponentials then run under the dP chain's matrix instructions, and
+                // the -rowsum(dO*O) values have the S chain's time to arrive from LDS (measured against the two chains
+                // interleaved step by step: -9 %)
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
+#pragma unroll
+                for (int s = 0; s < 4; s++)
+                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int rr = 32 * qb + g * 8 + half * 4;
@@ -831,19 +852,21 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                         if ((r >> 2) * 8 + (r & 3) + dl < lim) sacc[r] = 0.f;
                 }
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);     // rowsum(dO*O) of the four queries, read where it is used
+                for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * pacc[r];
+                // dV needs only P, dK needs dS: the dV matrix instructions go first and run under the vector work that forms dS
 #pragma unroll
-                    for (int e = 0; e < 4; e++) pacc[4 * g + e] = sacc[4 * g + e] * (pacc[4 * g + e] - d4[e]);
+                for (int s2 = 0; s2 < 2; s2++) {
+                    const bf16x8 pf = pack_acc(sacc, s2);
+#pragma unroll
+                    for (int d = 0; d < 2; d++)
+                        dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
                 }
 #pragma unroll
                 for (int s2 = 0; s2 < 2; s2++) {
-                    const bf16x8 pf = pack_acc(sacc, s2), dsf = pack_acc(pacc, s2);
+                    const bf16x8 dsf = pack_acc(pacc, s2);
 #pragma unroll
-                    for (int d = 0; d < 2; d++) {
-                        dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
+                    for (int d = 0; d < 2; d++)
                         dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tq, laq, 32 * qb + 16 * s2, 32 * d), dsf, dk[d], 0, 0, 0);
-                    }
                 }
             }
             fa_tiles_landed();

@@ -90,8 +90,8 @@ constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 // Switch for a measured alternative, off in the product: the last K stage of a tile taken one 32-row block at a time, each
 // finished block's epilogue (strip pass and stores) placed behind the matrix instructions of the next block, the barrier and
 // the tile change before the last block. Bit-exact; it needs 20 more registers (253-255) and, timed against the product on
-// one machine, alternating: NT bias kernels +2 to +5 % (fc 0.340 -> 0.347 ms, fcproj 0.275 -> 0.290, qkv 0.210 -> 0.219), NT
-// GELU +1 to +3 %, NN store within +-1 %. python llm.c_amd/build.py --variant rowwise -DLLMK_ROWWISE_LAST=1 builds it for
+// one machine, both libraries loaded in one process and called in turn: NT bias kernels +2 to +7 % (fc 0.299 -> 0.315 ms,
+// fcproj 0.266 -> 0.285, qkv 0.206 -> 0.217), NT GELU +3 to +5 %, NN store within +-1 %, NN GELU backward +20 %. python llm.c_amd/build.py --variant rowwise -DLLMK_ROWWISE_LAST=1 builds it for
 // llm.c_amd/microbench.py --variant rowwise (2: also the GELU-backward kernels).
 #ifndef LLMK_ROWWISE_LAST
 #define LLMK_ROWWISE_LAST 0
