@@ -193,6 +193,16 @@ class LibraryMissing(RuntimeError):
 _loaded = {}
 
 
+def bind(lib):
+    """Types every entry point of an opened library (include/llmk.h, llmk_gpt2.h) and returns it."""
+    for table in (KERNEL_ABI, DRIVER_ABI, DATA_ABI):
+        for name, (res, args) in table.items():
+            fn = getattr(lib, name)   # AttributeError here = header and library disagree
+            fn.restype = res
+            fn.argtypes = args
+    return lib
+
+
 def load(precision="bf16"):
     """Loads lib/libllmk_<precision>.so and types every entry point. Raises if it is not built."""
     if precision not in ("bf16", "fp32"):
@@ -203,12 +213,7 @@ def load(precision="bf16"):
     if not os.path.exists(path):
         raise LibraryMissing(f"{path} not found: build it with `python llm.c_amd/build.py` "
                              "(there is no fallback implementation)")
-    lib = C.CDLL(path)
-    for table in (KERNEL_ABI, DRIVER_ABI, DATA_ABI):
-        for name, (res, args) in table.items():
-            fn = getattr(lib, name)   # AttributeError here = header and library disagree
-            fn.restype = res
-            fn.argtypes = args
+    lib = bind(C.CDLL(path))
     got = lib.llmk_precision().decode()
     if got != precision:
         raise RuntimeError(f"{path} reports precision {got}")

@@ -7,7 +7,12 @@ events on the launch stream (llmk_profile_*), so a case that launches several ke
 dweight GEMM, split-K reduce, bias gradient) reports each of them. Inputs are N(0,1) from a fixed seed, weights
 N(0,0.02). Before each repetition 1 GiB is overwritten, which evicts the 8 x 4 MiB L2s and the 256 MiB Infinity Cache.
 
-    python llm.c_amd/microbench.py [--reps 20] [--only gemm,attention,...] [--json out.json] [--variant NAME]
+    python llm.c_amd/microbench.py [--reps 20] [--only gemm,attention,...] [--json out.json] [--variant NAME | --against NAME[,NAME...]]
+
+--against loads the product library AND the named variant builds (lib/variants/NAME/, python llm.c_amd/build.py --variant
+NAME -D...) into this one process and calls them in turn, repetition by repetition, on the same buffers: differences between
+two builds of a kernel then show to about half a percent, where separate processes (or separate machines of the pool)
+differ by several percent in clock, memory placement and temperature.
 
 Prints, per kernel family and case: median and minimum milliseconds, the algorithmic TFLOP/s or GB/s at the median,
 and the fraction of the roofline that bounds the family (2500 TFLOP/s bf16 MFMA, 8000 GB/s HBM). PyTorch is used
@@ -34,10 +39,23 @@ PEAK_TFLOPS, PEAK_GBS = 2500.0, 8000.0
 MFMA_FAMILIES = ("gemm", "attention_forward", "attention_backward_dq", "attention_backward_dkdv")
 
 
-def run_cases(L, reps=20, only=(), emit=print):
+class _InTurn:
+    """Stands for whichever of several loaded libraries has the turn: the cases call through it."""
+
+    def __init__(self, lib):
+        self.cur = lib
+
+    def __getattr__(self, name):
+        return getattr(self.cur, name)
+
+
+def run_cases(L, reps=20, only=(), emit=print, others=()):
     """Runs every case (or those whose tag contains one of `only`) on the loaded library L and returns the list of
-    per-kernel records. `emit` receives the printed lines (None: silent)."""
+    per-kernel records. `emit` receives the printed lines (None: silent). `others`: (tag, library) pairs timed in turn
+    with L in every repetition; their medians go into each record's "against"."""
     only = list(only)
+    turns = [("", L)] + list(others)
+    L = _InTurn(L)
     dev = "cuda"
     p = lambda t: None if t is None else C.c_void_p(t.data_ptr())
     g = torch.Generator(device=dev); g.manual_seed(1234)
@@ -48,35 +66,44 @@ def run_cases(L, reps=20, only=(), emit=print):
     calls, ms, fl, by = C.c_int(), C.c_double(), C.c_double(), C.c_double()
 
     def measure(fn, prepare=None):
-        """-> {family: (list of ms per rep, flops per rep, bytes per rep, launches per rep)}"""
+        """-> {family: (list of ms per rep, flops per rep, bytes per rep, launches per rep, {tag: list of ms})}"""
         out = {}
-        fn(); torch.cuda.synchronize()                        # warm-up (workspace growth, attribute setting)
+        for _, lib in turns:
+            L.cur = lib
+            fn(); torch.cuda.synchronize()                    # warm-up (workspace growth, attribute setting)
         for _ in range(reps):
-            if prepare: prepare()
-            flush_buf.zero_(); torch.cuda.synchronize()
-            L.llmk_profile_reset(); L.llmk_profile_enable(1)
-            fn()
-            torch.cuda.synchronize(); L.llmk_profile_enable(0)
-            for i in range(L.llmk_profile_count()):
-                L.llmk_profile_get(i, name, C.byref(calls), C.byref(ms), C.byref(fl), C.byref(by))
-                rec = out.setdefault(name.value.decode(), ([], fl.value, by.value, calls.value))
-                rec[0].append(ms.value)
+            for tag, lib in turns:
+                L.cur = lib
+                if prepare: prepare()
+                flush_buf.zero_(); torch.cuda.synchronize()
+                L.llmk_profile_reset(); L.llmk_profile_enable(1)
+                fn()
+                torch.cuda.synchronize(); L.llmk_profile_enable(0)
+                for i in range(L.llmk_profile_count()):
+                    L.llmk_profile_get(i, name, C.byref(calls), C.byref(ms), C.byref(fl), C.byref(by))
+                    rec = out.setdefault(name.value.decode(), ([], fl.value, by.value, calls.value, {}))
+                    (rec[4].setdefault(tag, []) if tag else rec[0]).append(ms.value)
+        L.cur = turns[0][1]
         return out
 
     results = []
 
     def report(case, out):
-        for fam, (times, flops, nbytes, ncalls) in out.items():
+        for fam, (times, flops, nbytes, ncalls, alt) in out.items():
             med, mn = statistics.median(times), min(times)
             mfma = fam.startswith(MFMA_FAMILIES)
             if mfma:
                 rate, unit, frac = flops / med * 1e-9, "TFLOP/s", flops / med * 1e-9 / PEAK_TFLOPS
             else:
                 rate, unit, frac = nbytes / med * 1e-6, "GB/s", nbytes / med * 1e-6 / PEAK_GBS
+            against = {tag: statistics.median(t) for tag, t in alt.items()}
             if emit:
-                emit(f"{case:34s} {fam:26s} x{ncalls:<2d} median {med:8.4f} ms  min {mn:8.4f} ms  {rate:9.1f} {unit:8s} {100 * frac:5.1f} % of {'MFMA' if mfma else 'HBM'} peak")
+                versus = "".join(f"  | {tag} {m:8.4f} ms {100 * (m / med - 1):+5.1f} %" for tag, m in against.items())
+                emit(f"{case:34s} {fam:26s} x{ncalls:<2d} median {med:8.4f} ms  min {mn:8.4f} ms  {rate:9.1f} {unit:8s} {100 * frac:5.1f} % of {'MFMA' if mfma else 'HBM'} peak{versus}")
             results.append({"case": case, "kernel": fam, "launches": ncalls, "median_ms": med, "min_ms": mn, "rate": rate, "unit": unit,
                             "bound": "mfma" if mfma else "hbm", "frac": frac, "flops": flops, "bytes": nbytes})
+            if against:
+                results[-1]["against"] = against
 
     def want(tag):
         return not only or any(o in tag for o in only)
@@ -203,12 +230,24 @@ def main():
     ap.add_argument("--json", default="")
     ap.add_argument("--variant", default="", help="time lib/variants/NAME/libllmk_bf16.so (python llm.c_amd/build.py --variant NAME "
                     "-D...: a build with ablation switches set, whose results are wrong by design) instead of the product library")
+    ap.add_argument("--against", default="", help="comma-separated variant names: time them in turn with the product library, in this process")
     args = ap.parse_args()
+    if args.variant and args.against:
+        ap.error("--variant replaces the product library, --against runs beside it: give one of them")
+    product_dir = pkg.LIBDIR
     if args.variant:
-        pkg.LIBDIR = os.path.join(pkg.LIBDIR, "variants", args.variant)
+        pkg.LIBDIR = os.path.join(product_dir, "variants", args.variant)
     L = pkg.load("bf16")          # raises LibraryMissing when the HIP library has not been built
     L.llmk_init(0)
-    results = run_cases(L, args.reps, [s for s in args.only.split(",") if s], lambda line: print(line, flush=True))
+    others = []
+    for tag in [t for t in args.against.split(",") if t]:
+        path = os.path.join(product_dir, "variants", tag, "libllmk_bf16.so")
+        if not os.path.exists(path):
+            raise pkg.LibraryMissing(f"{path} not found: python llm.c_amd/build.py --variant {tag} -D...")
+        lib = pkg.bind(C.CDLL(path))
+        lib.llmk_init(0)
+        others.append((tag, lib))
+    results = run_cases(L, args.reps, [s for s in args.only.split(",") if s], lambda line: print(line, flush=True), others)
     if args.json:
         with open(args.json, "w") as f:
             json.dump({"reps": args.reps, "peak_tflops": PEAK_TFLOPS, "peak_gbs": PEAK_GBS, "results": results}, f, indent=1)
