@@ -387,3 +387,40 @@ def test_attention_exact_zeros(zero):
     for i in ((0, 2) if zero == "Q" else (1, 2)):
         assert rel_fro(d[:, :, i], rd[:, :, i]) < 1e-2, i
     G.check_no_error(L)
+
+
+def test_row_wise_last_stage_variant_gives_the_same_bits():
+    """The GEMM kernel's switched-off alternative schedule (LLMK_ROWWISE_LAST, a variant build that
+    llm.c_amd/microbench.py --against rowwise times) changes the order of instructions, not of additions: where that
+    build is present it must agree with the product library bit for bit, forward (bias and GELU epilogues) and dinp."""
+    import os
+    import torch
+    pkg = G.package()
+    path = os.path.join(os.path.dirname(pkg.lib_path("bf16")), "variants", "rowwise", "libllmk_bf16.so")
+    if not os.path.exists(path):
+        pytest.skip("no variant build: python llm.c_amd/build.py bf16 --variant rowwise -DLLMK_ROWWISE_LAST=1")
+    L = G.lib("bf16")
+    V = pkg.bind(CT.CDLL(path))
+    V.llmk_init(0)
+    g = torch.Generator(device="cuda"); g.manual_seed(11)
+    rn = lambda *s, scale=1.0: (torch.randn(*s, device="cuda", generator=g) * scale).to(torch.bfloat16)
+    for C, OC in ((768, 3072), (3072, 768), (768, 2000)):          # the last one: tiles that reach past N
+        M = N_ROWS // 2
+        x, w, b = rn(M, C), rn(OC, C, scale=0.05), rn(OC)
+        outs = []
+        for lib in (L, V):
+            out = torch.full((M, OC), 3.0, dtype=torch.bfloat16, device="cuda")
+            pre = torch.full((M, OC), 5.0, dtype=torch.bfloat16, device="cuda")
+            act = torch.full((M, OC), 5.0, dtype=torch.bfloat16, device="cuda")
+            lib.llmk_matmul_forward(G.ptr(out), G.ptr(x), G.ptr(w), G.ptr(b), 1, M, C, OC, None, None, 1)
+            lib.llmk_matmul_forward(G.ptr(act), G.ptr(x), G.ptr(w), G.ptr(b), 1, M, C, OC, None, G.ptr(pre), 2)
+            dinp = torch.full((M, C), 3.0, dtype=torch.bfloat16, device="cuda")
+            dw = torch.zeros((OC, C), dtype=torch.bfloat16, device="cuda")
+            lib.llmk_matmul_backward(G.ptr(dinp), G.ptr(dw), None, G.ptr(out), G.ptr(x), G.ptr(w), None, 1, M, C, OC, None, None, 1)
+            G.sync()
+            outs.append((out, pre, act, dinp, dw))
+        for a, c, what in zip(outs[0], outs[1], ("forward", "pre-activation", "activation", "dinp", "dweight")):
+            assert torch.isfinite(a.float()).all()
+            assert torch.equal(a, c), (C, OC, what)
+    G.check_no_error(L)
+    assert V.llmk_last_error() in (None, b"")
