@@ -3,11 +3,13 @@
 with the reference's CPU trainer timed beside it.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu-baseline] [--no-kernel-events] [--no-mfma-probe]
-                    [--no-other-configs] [--no-microbench] [--model d12|d24|d48 --batch B --recompute R]
+                    [--no-other-configs] [--no-microbench] [--model d12|d24|d48 --batch B --recompute R] [--reference-loop]
 
 A step = gpt2_forward + gpt2_backward_and_reduce + gpt2_calculate_grad_norm (clip at 1.0) + gpt2_update
 on one batch of synthetic tokens, exactly the work of one iteration of the reference's training loop
-(train_gpt2.cu:1829-1852) with grad_accum_steps = 1. Prints one JSON line.
+(train_gpt2.cu:1829-1852) with grad_accum_steps = 1, queued as a whole by gpt2_train_step (same kernels, same results
+bit for bit; the host waits for the device once per step instead of four times). --reference-loop makes the four
+calls instead. Prints one JSON line.
 """
 import argparse
 import ctypes as C
@@ -155,7 +157,7 @@ def default_headline(args):
     return (args.batch, args.seq, args.model, args.recompute, args.gelu_fusion) == (64, 1024, "d12", 0, 3)
 
 
-def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, kernel_events, lr=6e-4):
+def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, kernel_events, lr=6e-4, reference_loop=False):
     """Builds the model, runs warmup + steps training steps on one synthetic batch, returns the result fields."""
     default_workload = (B, T, model, recompute, gelu_fusion) == (64, 1024, "d12", 0, 3)
     h = L.gpt2_create()
@@ -171,14 +173,20 @@ def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, k
     inp, tgt = np.ascontiguousarray(stream[:-1]), np.ascontiguousarray(stream[1:])
     ip, tp = inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p)
 
+    loss_f, norm_f = C.c_float(), C.c_float()
+
     def step(t):
-        L.gpt2_forward(h, ip, B, T)
-        L.gpt2_backward_and_reduce(h, ip, tp, 1, 0)
-        loss = L.gpt2_mean_loss(h)
-        norm = L.gpt2_calculate_grad_norm(h)
-        scale = 1.0 / norm if norm > 1.0 else 1.0
-        L.gpt2_update(h, lr, 0.9, 0.95, 1e-8, 0.1, scale, t, 0)
-        return loss, norm
+        if reference_loop:                   # the reference's four calls, each waiting for the device (train_gpt2.cu:1835-1851)
+            L.gpt2_forward(h, ip, B, T)
+            L.gpt2_backward_and_reduce(h, ip, tp, 1, 0)
+            loss = L.gpt2_mean_loss(h)
+            norm = L.gpt2_calculate_grad_norm(h)
+            scale = 1.0 / norm if norm > 1.0 else 1.0
+            L.gpt2_update(h, lr, 0.9, 0.95, 1e-8, 0.1, scale, t, 0)
+            return loss, norm
+        # the same step queued as a whole: same kernels, same bits, one wait at the end
+        L.gpt2_train_step(h, ip, tp, lr, 0.9, 0.95, 1e-8, 0.1, 1.0, t, C.byref(loss_f), C.byref(norm_f))
+        return loss_f.value, norm_f.value
 
     def read_profile(nsteps):
         recs = []
@@ -258,7 +266,8 @@ def run_workload(L, torch, model, B, T, recompute, gelu_fusion, steps, warmup, k
                                {("d12", 64, 1024): " (BASELINE configs[2])", ("d24", 32, 1024): " (BASELINE configs[3])",
                                 ("d48", 16, 1024): " (BASELINE configs[4])"}.get((model, B, T), ""),
                    "global_batch": B, "seq_len": T, "tokens_per_step": B * T, "recompute": recompute,
-                   "gelu_fusion": gelu_fusion, "parallelism": "single GPU"},
+                   "gelu_fusion": gelu_fusion, "parallelism": "single GPU",
+                   "step_calls": "reference loop (4 calls, 4 waits)" if reference_loop else "gpt2_train_step (1 wait)"},
         "mfu": float(mfu), "mfu_peak_tflops": PEAK_BF16_TFLOPS,
         "loss_first": float(losses[0]), "loss_last": float(losses[-1]), "losses": [round(float(x), 4) for x in losses],
         "roofline": roofline, "kernels_from_last_warmup_step": kernels,
@@ -277,6 +286,8 @@ def main():
     # 3: GELU in both GEMM epilogues with gelu'(pre-activation) kept for the backward one (this library's own level; the
     # reference's highest is 2, which --gelu-fusion 2 runs)
     ap.add_argument("--gelu-fusion", type=int, default=3)
+    ap.add_argument("--reference-loop", action="store_true",
+                    help="drive the step by the reference's four calls (each waits for the device) instead of gpt2_train_step")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-events", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true")
@@ -316,7 +327,7 @@ def main():
 
     with SclkSampler() as step_clock:
         out = run_workload(L, torch, args.model, args.batch, args.seq, args.recompute, args.gelu_fusion, args.steps,
-                           args.warmup, not args.no_kernel_events)
+                           args.warmup, not args.no_kernel_events, reference_loop=args.reference_loop)
     out = {"metric": METRIC, **out}
 
     if not args.no_mfma_probe:
@@ -351,7 +362,7 @@ def main():
         # own recipe (scripts/run_gpt2_350M.sh:29-34: -b 64; scripts/run_gpt2_1558M.sh:27-33 has -b 16). No recomputation
         # (-r 0) and the learning rates of those recipes.
         for model, b, lr in (("d24", 32, 3e-4), ("d48", 16, 6e-4), ("d24", 64, 3e-4)):
-            r = run_workload(L, torch, model, b, 1024, 0, args.gelu_fusion, 3, 2, False, lr=lr)
+            r = run_workload(L, torch, model, b, 1024, 0, args.gelu_fusion, 3, 2, False, lr=lr, reference_loop=args.reference_loop)
             out["other_configs"].append({k: r[k] for k in ("value", "unit", "ms_per_step", "mfu", "steps", "warmup", "config",
                                                               "loss_first", "loss_last", "losses")})
     if default_headline(args) and not args.no_microbench:

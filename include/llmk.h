@@ -258,6 +258,15 @@ int llmk_adamw_update_multi(void* params_memory, float* master, const void* grad
                             const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
                             const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
                             void* stream);
+/* The same launch with the clipping decided on the device: grad_scale = norm > grad_clip ? grad_clip / norm : 1 with
+ * norm = sqrt(*grad_norm_squared) (device memory: the result of llmk_global_norm_squared + llmk_global_sum_deterministic),
+ * the two statements of the reference's training loop (train_gpt2.cu:1841-1851) in the same fp32 arithmetic. No
+ * counterpart in the reference: for step loops that do not want to wait for the norm on the host between the backward
+ * pass and the update. Returns 0 (nothing launched) where llmk_adamw_update_multi would. */
+int llmk_adamw_update_multi_clip(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                                 const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                                 const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps,
+                                 const float* grad_norm_squared, float grad_clip, void* stream);
 
 /* init_from_master, llmc/adamw.cuh:90. params = stochastic_round(master), same noise as above. */
 void llmk_init_from_master(void* params_memory, const float* master_params_memory, size_t num_parameters,

@@ -55,6 +55,14 @@ float gpt2_calculate_grad_norm(LLMK_GPT2* m);
 /* gpt2_update, train_gpt2.cu:1035 */
 void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, float eps, float weight_decay,
                  float grad_scale, int t, int init_from_master_only);
+/* One optimizer step over one micro-batch with a single wait at its end: gpt2_forward + gpt2_backward_and_reduce(.., 1, 0)
+ * + gpt2_calculate_grad_norm + gpt2_update with grad_scale = norm > grad_clip ? grad_clip / norm : 1 (train_gpt2.cu:1835-1851),
+ * queued back to back, the clipping factor formed on the device, the mean loss and the gradient norm read back together
+ * after the update is queued. Same kernels in the same order on the same data: the parameters, the loss and the norm are
+ * those of the four calls, bit for bit. No counterpart in the reference (whose loop waits for the device after the forward
+ * pass, after the backward pass, for the norm and after the update). mean_loss / grad_norm may be NULL. */
+void gpt2_train_step(LLMK_GPT2* m, const int* inputs, const int* targets, float learning_rate, float beta1, float beta2,
+                     float eps, float weight_decay, float grad_clip, int t, float* mean_loss, float* grad_norm);
 /* gpt2_estimate_mfu, train_gpt2.cu:1126, against the MI355X dense peak of the library's precision */
 float gpt2_estimate_mfu(LLMK_GPT2* m, int num_tokens, float dt);
 /* gpt2_free, train_gpt2.cu:1155 */

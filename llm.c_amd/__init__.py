@@ -80,6 +80,8 @@ KERNEL_ABI = {
     "llmk_adamw_update": (None, [vp, vp, vp, vp, vp, sz, pd, pd, pd, i32, f32, f32, f32, i32, f32, f32, f32, u32, vp]),
     "llmk_adamw_update_multi": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, i32,
                                       C.c_float, C.c_float, vp]),
+    "llmk_adamw_update_multi_clip": (i32, [vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, C.c_float, C.c_float, C.c_float, i32,
+                                           C.c_float, vp, C.c_float, vp]),
     "llmk_init_from_master": (None, [vp, vp, sz, pd, pd, i32, u32, vp]),
     "llmk_copy_and_cast_to_f32": (None, [vp, vp, sz, pd, pd, i32, vp]),
 }
@@ -98,6 +100,7 @@ DRIVER_ABI = {
     "gpt2_backward_and_reduce": (None, [vp, vp, vp, i32, i32]),
     "gpt2_calculate_grad_norm": (f32, [vp]),
     "gpt2_update": (None, [vp, f32, f32, f32, f32, f32, f32, i32, i32]),
+    "gpt2_train_step": (None, [vp, vp, vp, f32, f32, f32, f32, f32, f32, i32, vp, vp]),
     "gpt2_estimate_mfu": (f32, [vp, i32, f32]),
     "gpt2_free": (None, [vp]),
     "gpt2_save_state": (None, [vp, C.c_char_p, i32]),

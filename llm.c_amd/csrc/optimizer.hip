@@ -88,7 +88,8 @@ struct AdamTensorTable {
 };
 __global__ void __launch_bounds__(256)
 adamw_multi_kernel(floatX* __restrict__ params, float* __restrict__ master, const floatX* __restrict__ grads,
-                   float* __restrict__ m, float* __restrict__ v, AdamTensorTable tab, AdamArgs a) {
+                   float* __restrict__ m, float* __restrict__ v, AdamTensorTable tab, AdamArgs a,
+                   const float* __restrict__ grad_norm_squared, float grad_clip) {
     int ti = 0;
     while (ti + 1 < tab.count && blockIdx.x >= tab.first_block[ti + 1]) ti++;      // wave-uniform, at most 15 steps
     const unsigned local = blockIdx.x - tab.first_block[ti];
@@ -99,6 +100,10 @@ adamw_multi_kernel(floatX* __restrict__ params, float* __restrict__ master, cons
     const size_t base = tab.offset[ti] + (size_t)slice * n + i;
     a.wd = tab.wd[ti];
     a.seed = tab.seed[ti];
+    if (grad_norm_squared) {              // clipping decided here: the host's two statements (train_gpt2.cu:1841-1851), correctly rounded alike
+        const float norm = sqrtf(*grad_norm_squared);
+        a.gscale = norm > grad_clip ? grad_clip / norm : 1.0f;
+    }
     vecX g = ld_vec_nt(grads + base);
     vecX p;
     if (!master) p = ld_vec(params + base);
@@ -237,10 +242,10 @@ void llmk_adamw_update(void* params_memory, float* master, const void* grads_mem
     LAUNCH_CHECK();
 }
 
-int llmk_adamw_update_multi(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
-                            const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
-                            const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
-                            void* stream) {
+static int adamw_multi(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                       const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                       const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
+                       const float* grad_norm_squared, float grad_clip, void* stream) {
     if (llmk::failed()) return 0;
     if (count <= 0 || count > AdamTensorTable::MAX) return 0;
     auto al = [](const void* p) { return ((uintptr_t)p % 16) == 0; };
@@ -262,9 +267,27 @@ int llmk_adamw_update_multi(void* params_memory, float* master, const void* grad
     AdamArgs a{lr, beta1, beta2, 1.0f - powf(beta1, (float)t), 1.0f - powf(beta2, (float)t), eps, 0.f, grad_scale, 0u};
     hipStream_t st = (hipStream_t)stream;
     llmk::ProfScope prof("adamw_update", 0, elems * (master ? 2.0 * sizeof(floatX) + 24.0 : 3.0 * sizeof(floatX) + 16.0), st);
-    adamw_multi_kernel<<<(unsigned)blocks, 256, 0, st>>>((floatX*)params_memory, master, (const floatX*)grads_memory, m, v, tab, a);
+    adamw_multi_kernel<<<(unsigned)blocks, 256, 0, st>>>((floatX*)params_memory, master, (const floatX*)grads_memory, m, v, tab, a,
+                                                         grad_norm_squared, grad_clip);
     LAUNCH_CHECK();
     return 1;
+}
+
+int llmk_adamw_update_multi(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                            const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                            const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps, float grad_scale,
+                            void* stream) {
+    return adamw_multi(params_memory, master, grads_memory, m, v, count, offsets, sizes, num_slices, weight_decays, seeds, lr, beta1,
+                       beta2, t, eps, grad_scale, nullptr, 0.f, stream);
+}
+
+int llmk_adamw_update_multi_clip(void* params_memory, float* master, const void* grads_memory, float* m, float* v, int count,
+                                 const size_t* offsets, const size_t* sizes, const int* num_slices, const float* weight_decays,
+                                 const unsigned int* seeds, float lr, float beta1, float beta2, int t, float eps,
+                                 const float* grad_norm_squared, float grad_clip, void* stream) {
+    if (grad_norm_squared == nullptr) return 0;
+    return adamw_multi(params_memory, master, grads_memory, m, v, count, offsets, sizes, num_slices, weight_decays, seeds, lr, beta1,
+                       beta2, t, eps, 1.0f, grad_norm_squared, grad_clip, stream);
 }
 
 void llmk_init_from_master(void* params_memory, const float* master, size_t n, ptrdiff_t w_stride,

@@ -420,7 +420,8 @@ void gpt2_allocate_state(LLMK_GPT2* m, int B, int T) {
     llmk_workspace_reserve(ws);
 }
 
-void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T) {
+namespace {
+void forward_impl(LLMK_GPT2* m, const int* inputs, size_t B, size_t T, bool wait) {
     if (m->params_memory == nullptr) { printf("Error: model was not initialized properly.\n"); exit(EXIT_FAILURE); }
     const size_t Vp = m->config.padded_vocab_size, L = m->config.num_layers, NH = m->config.num_heads,
                  C = m->config.channels, X = m->X;
@@ -476,8 +477,11 @@ void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T) {
         }
     }
     llmk_matmul_forward(a.output, a.lnf, p.wte, nullptr, (int)B, (int)T, (int)C, (int)Vp, st, nullptr, 1);
-    hipCheck(hipStreamSynchronize(st));
+    if (wait) hipCheck(hipStreamSynchronize(st));
 }
+}  // namespace
+
+void gpt2_forward(LLMK_GPT2* m, const int* inputs, size_t B, size_t T) { forward_impl(m, inputs, B, T, true); }
 
 float gpt2_validate(LLMK_GPT2* m, const int* inputs, const int* targets, size_t B, size_t T) {
     assert(targets != nullptr);
@@ -520,7 +524,9 @@ void gpt2_generate(LLMK_GPT2* m, int* gen_tokens, int genT, int eot_token, unsig
     }
 }
 
-void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* targets, int grad_accum_steps, int micro_step) {
+namespace {
+// wait = false: everything is queued and nothing read back; the loss sum of the last micro-step stays in accumulated_mean_loss
+void backward_impl(LLMK_GPT2* m, const int* inputs, const int* targets, int grad_accum_steps, int micro_step, bool wait) {
     if (m->grads_memory == nullptr) { fprintf(stderr, "Need to allocate gradients before backward"); exit(EXIT_FAILURE); }
     const bool last_step = micro_step == grad_accum_steps - 1;
     hipStream_t st = m->stream;
@@ -588,30 +594,46 @@ void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* target
     }
     llmk_encoder_backward(g.wte, g.wpe, a.output, m->workload_indices, m->bucket_info, dresidual, m->inputs, inputs,
                           (int)B, (int)T, (int)C, llmk::random_u32(&m->rng_state), st);
-    if (last_step) {
-        llmk_global_sum_deterministic(m->accumulated_mean_loss, a.losses, (int)(B * T), st);
-        hipCheck(hipMemcpyAsync(&m->mean_loss, m->accumulated_mean_loss, sizeof(float), hipMemcpyDeviceToHost, st));
-    }
+    if (last_step) llmk_global_sum_deterministic(m->accumulated_mean_loss, a.losses, (int)(B * T), st);
+    if (!wait) return;
+    if (last_step) hipCheck(hipMemcpyAsync(&m->mean_loss, m->accumulated_mean_loss, sizeof(float), hipMemcpyDeviceToHost, st));
     hipCheck(hipStreamSynchronize(st));
     if (last_step) m->mean_loss /= (float)(B * T * grad_accum_steps);
     else m->mean_loss = -1.0f;
 }
+}  // namespace
 
-float gpt2_calculate_grad_norm(LLMK_GPT2* m) {
+void gpt2_backward_and_reduce(LLMK_GPT2* m, const int* inputs, const int* targets, int grad_accum_steps, int micro_step) {
+    backward_impl(m, inputs, targets, grad_accum_steps, micro_step, true);
+}
+
+namespace {
+// the squared norm of all gradients, left in the first float of the logits buffer (free after the backward pass)
+float* launch_grad_norm_squared(LLMK_GPT2* m) {
     hipStream_t st = m->stream;
     float* grad_norm_squared = (float*)m->acts.output;
     int num_slices[2] = {1, m->config.num_layers};
     int max_num_block_sums = llmk_get_max_num_block_sums(num_slices, 2);
     llmk_global_norm_squared(grad_norm_squared, m->grads_memory, m->num_parameters, 0, 1, max_num_block_sums, 1, st);
     llmk_global_sum_deterministic(grad_norm_squared, grad_norm_squared, max_num_block_sums, st);
+    return grad_norm_squared;
+}
+}  // namespace
+
+float gpt2_calculate_grad_norm(LLMK_GPT2* m) {
+    hipStream_t st = m->stream;
+    float* grad_norm_squared = launch_grad_norm_squared(m);
     float cpu = 0.0f;
     hipCheck(hipMemcpyAsync(&cpu, grad_norm_squared, sizeof(float), hipMemcpyDeviceToHost, st));
     hipCheck(hipStreamSynchronize(st));
     return sqrtf(cpu);
 }
 
-void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, float eps, float weight_decay,
-                 float grad_scale, int t, int init_from_master_only) {
+namespace {
+// grad_norm_squared given: the clipping factor is formed on the device from it and grad_clip (grad_scale unused), and the
+// call returns 0 without launching anything when the one-launch update does not take this model. wait = false: queued only.
+int update_impl(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, float eps, float weight_decay,
+                float grad_scale, const float* grad_norm_squared, float grad_clip, int t, int init_from_master_only, bool wait) {
     if (m->grads_memory == nullptr || m->m_memory == nullptr || m->v_memory == nullptr) {
         fprintf(stderr, "Need to allocate optimizer state before update");
         exit(EXIT_FAILURE);
@@ -639,14 +661,20 @@ void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, fl
             slices[i] = (i < 2 || i > 13) ? 1 : m->config.num_layers;
             wds[i] = (i == 0 || i == 1 || i == 4 || i == 6 || i == 10 || i == 12) ? weight_decay : 0.0f;
         }
-        if (llmk_adamw_update_multi(m->params_memory, m->master_weights, m->grads_memory, m->m_memory, m->v_memory,
-                                    NUM_PARAMETER_TENSORS, offsets, sizes, slices, wds, seeds, learning_rate, beta1, beta2, t,
-                                    eps, grad_scale, st)) {
+        const int launched = grad_norm_squared
+            ? llmk_adamw_update_multi_clip(m->params_memory, m->master_weights, m->grads_memory, m->m_memory, m->v_memory,
+                                           NUM_PARAMETER_TENSORS, offsets, sizes, slices, wds, seeds, learning_rate, beta1, beta2, t,
+                                           eps, grad_norm_squared, grad_clip, st)
+            : llmk_adamw_update_multi(m->params_memory, m->master_weights, m->grads_memory, m->m_memory, m->v_memory,
+                                      NUM_PARAMETER_TENSORS, offsets, sizes, slices, wds, seeds, learning_rate, beta1, beta2, t,
+                                      eps, grad_scale, st);
+        if (launched) {
             m->rng_state = rng;
-            hipCheck(hipStreamSynchronize(st));
-            return;
+            if (wait) hipCheck(hipStreamSynchronize(st));
+            return 1;
         }
     }
+    if (grad_norm_squared) return 0;       // the per-tensor launches below take their factor from the host
     for (int i = 0; i < NUM_PARAMETER_TENSORS; i++) {
         unsigned int seed = llmk::random_u32(&m->rng_state);
         int num_layers = (i < 2 || i > 13) ? 1 : m->config.num_layers;
@@ -668,7 +696,52 @@ void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, fl
                               eps, wd, grad_scale, seed, st);
         }
     }
+    if (wait) hipCheck(hipStreamSynchronize(st));
+    return 1;
+}
+}  // namespace
+
+void gpt2_update(LLMK_GPT2* m, float learning_rate, float beta1, float beta2, float eps, float weight_decay,
+                 float grad_scale, int t, int init_from_master_only) {
+    update_impl(m, learning_rate, beta1, beta2, eps, weight_decay, grad_scale, nullptr, 0.f, t, init_from_master_only, true);
+}
+
+// One optimizer step (one micro-batch) with a single wait at its end: forward, backward, gradient norm, clipping and
+// update are queued back to back, the clipping factor is formed on the device, and the loss and the norm come back
+// together after the update has been queued. The same kernels on the same data as gpt2_forward +
+// gpt2_backward_and_reduce(.., 1, 0) + gpt2_calculate_grad_norm + gpt2_update with the factor of train_gpt2.cu:1850, so the
+// same bits; what is gone are the four places where the GPU waits for the host (the reference's loop has them:
+// train_gpt2.cu:785, :975, :1021, :1148). No counterpart in the reference.
+void gpt2_train_step(LLMK_GPT2* m, const int* inputs, const int* targets, float learning_rate, float beta1, float beta2,
+                     float eps, float weight_decay, float grad_clip, int t, float* mean_loss, float* grad_norm) {
+    const size_t B = m->batch_size, T = m->seq_len;
+    hipStream_t st = m->stream;
+    forward_impl(m, inputs, B, T, false);
+    backward_impl(m, inputs, targets, 1, 0, false);
+    // the first-step work of gpt2_update that has to precede the norm's use of the logits buffer: none; the moments are
+    // cleared and the master copy taken inside update_impl, after the norm
+    const bool first = m->init_state;
+    float* norm2 = launch_grad_norm_squared(m);
+    float gn = -1.0f;
+    bool fused = false;
+    if (!(first && m->master_weights != nullptr))
+        fused = update_impl(m, learning_rate, beta1, beta2, eps, weight_decay, 1.0f, norm2, grad_clip, t, 0, false) != 0;
+    if (!fused) {                                // first step with a master copy to take, or a model the one-launch update does not take
+        float cpu = 0.0f;
+        hipCheck(hipMemcpyAsync(&cpu, norm2, sizeof(float), hipMemcpyDeviceToHost, st));
+        hipCheck(hipStreamSynchronize(st));
+        gn = sqrtf(cpu);
+        const float scale = (gn > grad_clip) ? grad_clip / gn : 1.0f;
+        update_impl(m, learning_rate, beta1, beta2, eps, weight_decay, scale, nullptr, 0.f, t, 0, false);
+    }
+    float* back = m->cpu_losses;                 // pinned
+    hipCheck(hipMemcpyAsync(&back[0], m->accumulated_mean_loss, sizeof(float), hipMemcpyDeviceToHost, st));
+    if (fused) hipCheck(hipMemcpyAsync(&back[1], norm2, sizeof(float), hipMemcpyDeviceToHost, st));
     hipCheck(hipStreamSynchronize(st));
+    m->mean_loss = back[0] / (float)(B * T);
+    if (fused) gn = sqrtf(back[1]);
+    if (mean_loss) *mean_loss = m->mean_loss;
+    if (grad_norm) *grad_norm = gn;
 }
 
 float gpt2_estimate_mfu(LLMK_GPT2* m, int num_tokens, float dt) {

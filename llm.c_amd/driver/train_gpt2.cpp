@@ -283,24 +283,35 @@ int main(int argc, char** argv) {
         // ---- one optimisation step over total_batch_size tokens ----
         if (overfit_single_batch == 1) dataloader_reset(train_loader);
         (void)hipEventRecord(start, nullptr);
-        for (int micro_step = 0; micro_step < grad_accum_steps; micro_step++) {
-            dataloader_next_batch(train_loader);
-            gpt2_forward(model, dataloader_inputs(train_loader), B, T);
-            gpt2_backward_and_reduce(model, dataloader_inputs(train_loader), dataloader_targets(train_loader), grad_accum_steps, micro_step);
-        }
-        const float mean_loss = gpt2_mean_loss(model);
-        const float zloss = (float)update_detector(loss_detector, (double)mean_loss);
+        float mean_loss, grad_norm, zloss, zgrad;
         const float step_learning_rate = get_learning_rate(sched, step);
-        const float grad_norm = gpt2_calculate_grad_norm(model);
-        const float zgrad = (float)update_detector(norm_detector, (double)grad_norm);
-        if (std::isfinite(zloss) && skip_update_lossz != 0.0f && zloss > skip_update_lossz) {
-            printf("skipping update due to loss z-score of %f\n", zloss);
-        } else if (std::isfinite(zgrad) && skip_update_gradz != 0.0f && zgrad > skip_update_gradz) {
-            printf("skipping update due to grad z-score of %f\n", zgrad);
+        if (grad_accum_steps == 1 && skip_update_lossz == 0.0f && skip_update_gradz == 0.0f) {
+            // nothing can veto the update and there is one micro-batch: the whole step is queued at once, the clipping
+            // factor is formed on the device, and the host waits once (same results as the calls below, bit for bit)
+            dataloader_next_batch(train_loader);
+            gpt2_train_step(model, dataloader_inputs(train_loader), dataloader_targets(train_loader), step_learning_rate, 0.9f, 0.95f,
+                            1e-8f, weight_decay, 1.0f, step + 1, &mean_loss, &grad_norm);
+            zloss = (float)update_detector(loss_detector, (double)mean_loss);
+            zgrad = (float)update_detector(norm_detector, (double)grad_norm);
         } else {
-            const float grad_clip = 1.0f;
-            const float grad_scale = grad_norm > grad_clip ? grad_clip / grad_norm : 1.0f;
-            gpt2_update(model, step_learning_rate, 0.9f, 0.95f, 1e-8f, weight_decay, grad_scale, step + 1, 0);
+            for (int micro_step = 0; micro_step < grad_accum_steps; micro_step++) {
+                dataloader_next_batch(train_loader);
+                gpt2_forward(model, dataloader_inputs(train_loader), B, T);
+                gpt2_backward_and_reduce(model, dataloader_inputs(train_loader), dataloader_targets(train_loader), grad_accum_steps, micro_step);
+            }
+            mean_loss = gpt2_mean_loss(model);
+            zloss = (float)update_detector(loss_detector, (double)mean_loss);
+            grad_norm = gpt2_calculate_grad_norm(model);
+            zgrad = (float)update_detector(norm_detector, (double)grad_norm);
+            if (std::isfinite(zloss) && skip_update_lossz != 0.0f && zloss > skip_update_lossz) {
+                printf("skipping update due to loss z-score of %f\n", zloss);
+            } else if (std::isfinite(zgrad) && skip_update_gradz != 0.0f && zgrad > skip_update_gradz) {
+                printf("skipping update due to grad z-score of %f\n", zgrad);
+            } else {
+                const float grad_clip = 1.0f;
+                const float grad_scale = grad_norm > grad_clip ? grad_clip / grad_norm : 1.0f;
+                gpt2_update(model, step_learning_rate, 0.9f, 0.95f, 1e-8f, weight_decay, grad_scale, step + 1, 0);
+            }
         }
         (void)hipEventRecord(end, nullptr);
         (void)hipEventSynchronize(end);

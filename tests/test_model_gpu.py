@@ -66,6 +66,12 @@ class Model:
         L.gpt2_update(h, lr, b1, b2, eps, wd, scale, t, 0)
         return loss, norm
 
+    def train_step(self, inp, tgt, t, lr, b1, b2, eps, wd, clip):
+        loss, norm = C.c_float(), C.c_float()
+        self.L.gpt2_train_step(self.h, inp.ctypes.data_as(C.c_void_p), tgt.ctypes.data_as(C.c_void_p), lr, b1, b2, eps, wd, clip, t,
+                               C.byref(loss), C.byref(norm))
+        return loss.value, norm.value
+
     def free(self):
         self.L.gpt2_free(self.h)
         self.h = None
@@ -214,6 +220,33 @@ def test_bf16_gpt2_124m_config0_tracks_cpu_loss(config0_oracle):
     wte = m.params()[:sizes[0]].reshape(cfg.padded_vocab_size, cfg.channels)
     assert (wte[cfg.vocab_size:] == 0).all()
     m.free()
+
+
+@pytest.mark.parametrize("master", [1, 0])
+@pytest.mark.parametrize("precision", ["bf16", "fp32"])
+def test_train_step_is_the_four_calls_bit_for_bit(precision, master):
+    """gpt2_train_step queues forward, backward, norm, clipping and update without waiting in between and forms the
+    clipping factor on the device; the loss, the gradient norm and every parameter must be those of the reference's four
+    calls (train_gpt2.cu:1835-1851), step after step - with a clip that bites (0.25 against norms near 1) and one that
+    does not (100), with and without the fp32 master copy (whose first step takes the host path), and interleaved with
+    the four calls on the same model."""
+    cfg = ol.Config(64, 300, 320, 2, 2, 128)
+    B, T = 4, 64
+    hp = (3e-3, 0.9, 0.95, 1e-8, 0.1)
+    for clip in (0.25, 100.0):
+        a = Model(precision, cfg, B, T, seed=5, master=master)
+        b = Model(precision, cfg, B, T, seed=5, master=master)
+        for s in range(5):
+            inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 20 + s)
+            want = a.step(inp, tgt, s + 1, *hp, clip=clip)
+            got = b.train_step(inp, tgt, s + 1, *hp, clip) if s != 3 else b.step(inp, tgt, s + 1, *hp, clip=clip)
+            assert got == want, (precision, master, clip, s, got, want)
+            if clip == 0.25:
+                assert want[1] > clip, "the clip is meant to bite"
+        np.testing.assert_array_equal(b.params(), a.params())
+        assert b.L.gpt2_mean_loss(b.h) == a.L.gpt2_mean_loss(a.h)
+        a.free(); b.free()
+    G.check_no_error(G.lib(precision))
 
 
 @pytest.mark.parametrize("precision", ["bf16", "fp32"])
@@ -450,17 +483,17 @@ def test_bf16_generation_samples_from_its_own_logits():
     m.free()
 
 
-def full_size_steps(cfg, B, T, recompute, gelu_fusion, steps=3, want_wte=True, lr=6e-4):
+def full_size_steps(cfg, B, T, recompute, gelu_fusion, steps=3, want_wte=True, lr=6e-4, whole_step=False):
     """A few AdamW steps at a shape the oracle cannot run, with what must hold at any size checked on the way: the
     initial loss (the final LayerNorm gives unit-variance channels and wte is N(0, 0.02), so the logits of a position
     are independent normals of variance s2 = 0.0004 * C, whose expected cross-entropy against a random target is
     ln(V) + s2 / 2), a finite positive gradient norm, a loss that decreases on a repeated batch, padded wte rows
-    untouched. Returns the (loss, norm) pairs."""
+    untouched. whole_step: each step through gpt2_train_step instead of the four calls. Returns the (loss, norm) pairs."""
     inp, tgt = ol.make_tokens(B, T, cfg.vocab_size, 99)
     m = Model("bf16", cfg, B, T, seed=42, recompute=recompute, gelu_fusion=gelu_fusion)
     out = []
     for s in range(steps):
-        loss, norm = m.step(inp, tgt, s + 1, lr, 0.9, 0.95, 1e-8, 0.1, clip=1.0)
+        loss, norm = (m.train_step if whole_step else m.step)(inp, tgt, s + 1, lr, 0.9, 0.95, 1e-8, 0.1, 1.0)
         assert np.isfinite(loss) and np.isfinite(norm) and norm > 0, (s, loss, norm)
         out.append((loss, norm))
     assert abs(out[0][0] - (np.log(cfg.vocab_size) + 0.0002 * cfg.channels)) < 0.05, out
@@ -488,6 +521,8 @@ def test_bf16_full_size_step_in_every_mode():
     assert runs[(0, 0)] == runs[(1, 0)] == runs[(2, 0)], runs
     assert runs[(0, 2)] == runs[(1, 2)], runs
     assert runs[(1, 3)] == runs[(1, 2)], runs               # fusion 3 with recomputation runs as fusion 2
+    # the step as the benchmark drives it: one call, one wait, the clipping factor formed on the device
+    assert full_size_steps(cfg, B, T, 0, 3, whole_step=True) == runs[(0, 3)], runs
     first = {mode: r[0][0] for mode, r in runs.items()}
     assert len(set(first.values())) == 1, first
     for mode, r in runs.items():
