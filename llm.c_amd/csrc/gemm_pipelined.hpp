@@ -510,36 +510,56 @@ gemm_pipelined_kernel(GemmArgs g) {
     };
 
 
-    // Bias of the wave's columns (EPI_BIAS, EPI_BIAS_GELU), fetched once per tile near its end: block j, quad q holds
-    // the four columns j*32 + 8q + 4*half + 0..3 of the wave tile, the ones the lane owns in the epilogue. Loads that
-    // the compiler issues are awaited with vmcnt(0), which also waits for every hand-issued tile load in flight; so
-    // they are placed in the one window in which this wave has none: from the start of the tile's last stage (the
-    // last-but-one stage ended with a wait for everything) until the wave requests the next tile's first stage, which
-    // these kernels do only after claiming the bias (bias_ready), half-way through the last stage. Tiles that reach past N take plain
-    // loads in the epilogue instead (the columns are tested there).
+    // Bias of the wave's columns (EPI_BIAS, EPI_BIAS_GELU*). The matrix cores add it, after the tile's last K stage: one more
+    // K step whose column-side operand holds bias[n] at k = 0 (lane n of the lower half-wave, element 0; zeros elsewhere)
+    // and whose row-side operand holds 1 at k = 0. bf16 x 1 is exact, so every accumulator gets its column's bias in one
+    // fp32 addition, as the epilogue's vector add gave it; that is TM x TN matrix instructions per tile while the matrix
+    // cores would idle anyway, in place of an unpack and an add per element of the epilogue (64 vector instructions per
+    // 32-row block), and two 2-byte loads per lane in place of eight 8-byte ones. Lanes past N, or a null bias, add zero:
+    // the epilogue has no bias code at all. The loads are ordinary loads, which the compiler awaits with vmcnt(0) - that
+    // also waits for every hand-issued tile load in flight - so they are placed in the one window in which this wave has
+    // none: from the start of the tile's last stage (the last-but-one stage ended with a wait for everything) until the
+    // wave requests the next tile's first stage, which these kernels do only after claiming the bias (bias_ready),
+    // half-way through the last stage.
     constexpr bool HAS_BIAS = (EPI == EPI_BIAS || epi_gelu_fwd(EPI));
-    bf16x4 biasv[HAS_BIAS ? TN : 1][4];
-    bool bias_fast = false;
+    unsigned biasw[HAS_BIAS ? TN : 1];   // bias of column j*32 + idx of the wave tile in the low 16 bits (lanes 0-31; 0 in lanes 32-63)
+    bool bias_lane[HAS_BIAS ? TN : 1];
     auto request_bias = [&](int n0) {
         if constexpr (HAS_BIAS) {
-            bias_fast = g.bias != nullptr && n0 + BN <= g.N;
-            // unconditional, so that the values stay in the registers they arrive in (a branch here makes the compiler
-            // copy them where the paths join, which needs them at once): without a usable bias the lanes read the
-            // first bytes of A, which are there, and the epilogue ignores what they got
-            const floatX* bp = bias_fast ? g.bias + n0 + wn * WTN + 4 * half : g.A + 4 * half;
 #pragma unroll
-            for (int j = 0; j < TN; j++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) biasv[j][q] = *reinterpret_cast<const bf16x4*>(bp + j * 32 + q * 8);
+            for (int j = 0; j < TN; j++) {
+                const int n = n0 + wn * WTN + j * 32 + idx;
+                bias_lane[j] = g.bias != nullptr && half == 0 && n < g.N;
+                // unconditional, so that the value stays in the register it arrives in: lanes without a bias read the first
+                // bytes of A, which are there, and drop what they got when they claim it
+                const floatX* bp = bias_lane[j] ? g.bias + n : g.A;
+                biasw[j] = *reinterpret_cast<const unsigned short*>(bp);
+            }
             asm volatile("" ::: "memory");                        // the loads stay here: nothing below may pull them down to their use
         }
     };
     auto bias_ready = [&]() {
         if constexpr (HAS_BIAS) {
 #pragma unroll
-            for (int j = 0; j < TN; j++)
+            for (int j = 0; j < TN; j++) {
+                asm volatile("" : "+v"(biasw[j]));
+                biasw[j] = bias_lane[j] ? biasw[j] : 0u;
+            }
+        }
+    };
+    // acc[i][*] += bias: the one-hot K step for the 32-row block i (after bias_ready)
+    auto add_bias = [&](auto ic) {
+        if constexpr (HAS_BIAS && !(LLMK_GEMM_ABL & 2)) {
+            constexpr int i = decltype(ic)::value;
+            union { unsigned u[4]; bf16x8 v; } one, bj;
+            one.u[0] = half == 0 ? 0x3F80u : 0u;                  // bf16 1.0 at k = 0
+            one.u[1] = one.u[2] = one.u[3] = 0u;
+            bj.u[1] = bj.u[2] = bj.u[3] = 0u;
 #pragma unroll
-                for (int q = 0; q < 4; q++) asm volatile("" : "+v"(biasv[j][q]));
+            for (int j = 0; j < TN; j++) {
+                bj.u[0] = biasw[j];
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bj.v, one.v, acc[i][j], 0, 0, 0);
+            }
         }
     };
 
@@ -569,20 +589,6 @@ gemm_pipelined_kernel(GemmArgs g) {
                             float v[4];
 #pragma unroll
                             for (int e = 0; e < 4; e++) v[e] = acc[i][j][4 * q + e];
-                            if (HAS_BIAS && bias_fast) {
-                                const bf16x4 b4 = biasv[HAS_BIAS ? j : 0][q];
-#pragma unroll
-                                for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
-                            } else if (HAS_BIAS) {
-                                if (g.bias) {
-                                    const int n = wn0 + nl;
-                                    if (n < g.N) {
-                                        bf16x4 b4 = *reinterpret_cast<const bf16x4*>(g.bias + n);
-#pragma unroll
-                                        for (int e = 0; e < 4; e++) v[e] += (float)b4[e];
-                                    }
-                                }
-                            }
                             char* dst = strip + idx * 128;
                             if (F32OUT) {                         // 16 bytes: chunk 2q + half
                                 f32x4 o = {v[0], v[1], v[2], v[3]};
@@ -812,6 +818,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                     bias_ready();
                     if (early0 && (HAS_BIAS || late)) issue_from(tile_base_n, 0, buf_idx(nst - 2));   // (the early waves of a kernel without bias: one stage ago)
                 }
+                add_bias(ic);
                 if constexpr (i >= 1) {
                     if (!(LLMK_GEMM_ABL & 8)) epi_block(std::integral_constant<int, i - 1>{});
                 }
@@ -835,6 +842,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             mma(fa0, fb0, S2{});
             await_frags(fa1, fb1, NoneYounger{});
             mma(fa1, fb1, S3{});
+            static_for<TM>([&](auto ic) { add_bias(ic); });
 
             // ---- request the next work item's first K blocks, then run the epilogue under them --------
             barrier_no_fence();                                  // every wave is done reading both buffers
