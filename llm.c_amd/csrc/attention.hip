@@ -670,12 +670,12 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
 #pragma unroll
                 for (int e = 0; e < 4; e++) pacc[4 * g + e] = d4[e];
             }
+            constexpr int LAG = 4;                               // the S chain first, then the dP chain (one loop: see fa_backward_dkdv_dma_kernel)
 #pragma unroll
-            for (int s = 0; s < 4; s++)
-                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
-#pragma unroll
-            for (int s = 0; s < 4; s++)
-                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s, lane), vf[s], pacc, 0, 0, 0);
+            for (int s = 0; s < 4 + LAG; s++) {
+                if (s < 4) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tq, 32 * qb, s, lane), kf[s], sacc, 0, 0, 0);
+                if (s >= LAG) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(frag_rows(tdo, 32 * qb, s - LAG, lane), vf[s - LAG], pacc, 0, 0, 0);
+            }
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 const int rr = 32 * qb + g * 8 + half * 4;
@@ -828,13 +828,14 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 }
                 // one chain after the other, S first: its exponentials then run under the dP chain's matrix instructions, and
                 // the -rowsum(dO*O) values have the S chain's time to arrive from LDS (measured against the two chains
-                // interleaved step by step: -9 %)
+                // interleaved step by step: -9 %). Written as ONE loop on purpose: two loops of four are fused by the
+                // compiler, which puts the chains back side by side.
+                constexpr int LAG = 4;                           // steps by which the dP chain runs behind the S chain
 #pragma unroll
-                for (int s = 0; s < 4; s++)
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
-#pragma unroll
-                for (int s = 0; s < 4; s++)
-                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s), vf[s], pacc, 0, 0, 0);
+                for (int s = 0; s < 4 + LAG; s++) {
+                    if (s < 4) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
+                    if (s >= LAG) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s - LAG), vf[s - LAG], pacc, 0, 0, 0);
+                }
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
                     const int rr = 32 * qb + g * 8 + half * 4;
