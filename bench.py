@@ -28,7 +28,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E, vendor figure
 METRIC = "train tokens/sec + MFU, GPT-2 124M bf16 B=64 T=1024, 1 MI355X"
 
 TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "train_step_gpt2_124M_b64_t1024_hbm_traffic.txt")
-KERNEL_SOURCES = ("gemm.hip", "gemm_pipelined.hpp", "common.hpp", "gelu.hpp")
+KERNEL_SOURCES = ("gemm.hip", "gemm_tn.hip", "gemm_pipelined.hpp", "common.hpp", "gelu.hpp")
 
 
 def kernel_sources_sha16():

@@ -289,8 +289,12 @@ void launch_pipelined_cfg(GemmArgs g, int splits, hipStream_t st) {
 }
 template <bool A_T, bool B_T, int EPI>
 void launch_pipelined(const GemmArgs& g, int splits, bool big, hipStream_t st) {
-    if (big) launch_pipelined_cfg<256, 256, 2, 4, A_T, B_T, EPI>(g, splits, st);
-    else launch_pipelined_cfg<128, 128, 2, 2, A_T, B_T, EPI>(g, splits, st);
+    if constexpr (A_T && B_T) {                          // the weight gradient's kernels: compiled in gemm_tn.hip
+        launch_pipelined_tn(g, splits, big, EPI, 0, st);
+    } else {
+        if (big) launch_pipelined_cfg<256, 256, 2, 4, A_T, B_T, EPI>(g, splits, st);
+        else launch_pipelined_cfg<128, 128, 2, 2, A_T, B_T, EPI>(g, splits, st);
+    }
 }
 // pipelined kernel when its preconditions hold, generic kernel otherwise
 template <bool A_T, bool B_T, int EPI>
@@ -875,20 +879,8 @@ void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* do
             g_last_split_kind = 2; g_last_split_pieces = slots;
             {
                 llmk::ProfScope prof("gemm_tn_splitk", 2.0 * M * (double)OC * C, tn_bytes, st);
-                constexpr int SMEM = gemmk::smem_bytes(256, 256, 8);
-                if (dbias_in_gemm) {
-                    g.rowsum = g.partial + mn * slots;            // [slots * parts][OC]
-                    auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL_ROWSUM>;
-                    static bool attr_set = false;
-                    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
-                    kern<<<G, 512, SMEM, st>>>(g);
-                } else {
-                    auto kern = gemm_pipelined_kernel<256, 256, 2, 4, true, true, EPI_PARTIAL>;
-                    static bool attr_set = false;
-                    if (!attr_set) { HIP_CHECK(hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM)); attr_set = true; }
-                    kern<<<G, 512, SMEM, st>>>(g);
-                }
-                LAUNCH_CHECK();
+                if (dbias_in_gemm) g.rowsum = g.partial + mn * slots;            // [slots * parts][OC]
+                launch_pipelined_tn(g, slots, true, dbias_in_gemm ? EPI_PARTIAL_ROWSUM : EPI_PARTIAL, G, st);
             }
             llmk::ProfScope prof("splitk_reduce", 0, (double)mn * slots * sizeof(float) + 2.0 * mn * sizeof(floatX), st);
             const unsigned main_blocks = (unsigned)CEIL_DIV(mn / 4, (size_t)256);

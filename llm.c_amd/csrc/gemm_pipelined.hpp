@@ -882,6 +882,12 @@ gemm_pipelined_kernel(GemmArgs g) {
 #endif  // __HIP_DEVICE_COMPILE__
 }
 
+// The kernels with both operands K-major (the weight gradient: EPI_ACCUM, EPI_PARTIAL, EPI_PARTIAL_ROWSUM) live in a
+// translation unit of their own, gemm_tn.hip, because they are compiled with another instruction-scheduling strategy
+// than the rest of the library (see llm.c_amd/build.py). grid = 0: the usual grid (one workgroup per CU, at most one per
+// work item); otherwise that many workgroups (the uneven split of K, whose schedule is derived from the grid size).
+void launch_pipelined_tn(GemmArgs g, int splits, bool big, int epi, int grid, hipStream_t st);
+
 #endif  // !LLMK_FP32
 
 }  // namespace gemmk
