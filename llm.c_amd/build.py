@@ -25,7 +25,12 @@ KERNEL_SOURCES = ["runtime.hip", "layernorm.hip", "gelu.hip", "encoder.hip", "cl
 # options of single files: the weight-gradient GEMM kernels take the compiler's "max-ilp" instruction scheduling (measured
 # per kernel family, each variant loaded beside the product in one process: these kernels -1.2 to -2.7 %, every other GEMM
 # kernel +2 to +8 %, attention forward -1.5 %, dQ 0, dK/dV +9 %)
-FILE_FLAGS = {"gemm_tn.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"]}
+# The other GEMM kernels and attention: the pre-register-allocation scheduler working bottom-up only (same method: dinp
+# GEMMs -2 to -3.7 % (K = 3072 and the LM head), forward GEMMs -0.4 to -2.2 %, the GELU epilogue kernels +0.5 %, attention
+# dK/dV -1.5 %, forward and dQ unchanged; top-down only: every GEMM kernel +10 to +19 %).
+FILE_FLAGS = {"gemm_tn.hip": ["-mllvm", "-amdgpu-sched-strategy=max-ilp"],
+              "gemm.hip": ["-mllvm", "-misched-prera-direction=bottomup"],
+              "attention.hip": ["-mllvm", "-misched-prera-direction=bottomup"]}
 DRIVER_SOURCES = ["gpt2.cpp", "data.cpp"]
 
 # -packed-fp32-ops off: this toolchain's packed fp32 instructions are not trusted on this hardware pool
