@@ -96,7 +96,10 @@ void llmk_encoder_forward(void* out, const int* inp, const void* wte, const void
  *                     the position list (same layout and bound as the reference, llmc/encoder.cuh:183-184,225-226)
  *   workload_indices  host, >= B*T ints         (reference sizes it B*T*G)
  *   bucket_info       host, >= B*T*G * 4 ints   (reference: one int4 per bucket)
- *   inp / inputs_cpu  the same tokens on device / host */
+ *   inp / inputs_cpu  the same tokens on device / host
+ * The two host lists are copied to the device by asynchronous copies on `stream`: where the caller gives pinned memory
+ * (the driver does) the call returns with the copies and the kernel queued, and the lists must not be written again
+ * before the stream has passed them; with pageable memory the copies are done when the call returns. */
 void llmk_encoder_backward(void* dwte, void* dwpe, void* scratch, int* workload_indices, int* bucket_info,
                            const void* dout, const int* inp, const int* inputs_cpu, int B, int T, int C,
                            unsigned int seed, void* stream);

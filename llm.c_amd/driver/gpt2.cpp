@@ -406,8 +406,10 @@ void gpt2_allocate_state(LLMK_GPT2* m, int B, int T) {
     hipCheck(hipMalloc((void**)&m->accumulated_mean_loss, sizeof(float)));
     hipCheck(hipHostMalloc((void**)&m->cpu_losses, (size_t)B * T * sizeof(float)));
     size_t ncg = ceil_div(m->config.channels, 64 * (16 / m->X));
-    m->workload_indices = (int*)malloc(sizeof(int) * (size_t)B * T * ncg);
-    m->bucket_info = (int*)malloc(sizeof(int) * 4 * (size_t)B * T * ncg);
+    // pinned: the copies of the sorted buckets to the device (llmk_encoder_backward) are then queued without a wait, and the
+    // kernel that reads them right behind
+    hipCheck(hipHostMalloc((void**)&m->workload_indices, sizeof(int) * (size_t)B * T * ncg));
+    hipCheck(hipHostMalloc((void**)&m->bucket_info, sizeof(int) * 4 * (size_t)B * T * ncg));
     hipCheck(hipMalloc((void**)&m->m_memory, m->num_parameters * sizeof(float)));
     hipCheck(hipMalloc((void**)&m->v_memory, m->num_parameters * sizeof(float)));
     if (m->use_master_weights == 1) hipCheck(hipMalloc((void**)&m->master_weights, m->num_parameters * sizeof(float)));
@@ -761,8 +763,8 @@ void gpt2_free(LLMK_GPT2* m) {
                    m->inputs, m->targets, m->accumulated_mean_loss};
     for (void* p : dev) if (p) (void)hipFree(p);
     if (m->cpu_losses) (void)hipHostFree(m->cpu_losses);
-    free(m->workload_indices);
-    free(m->bucket_info);
+    if (m->workload_indices) (void)hipHostFree(m->workload_indices);
+    if (m->bucket_info) (void)hipHostFree(m->bucket_info);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
