@@ -722,9 +722,14 @@ gemm_pipelined_kernel(GemmArgs g) {
         for (int st = 0; st < nst - 1; st++) {
             const unsigned cur = buf_of(st);
             read_frags(cur, S1{}, fa1, fb1);
+            // where the late waves request the next stage: behind the step's first matrix instructions, or - the kernels
+            // with both operands K-major - ahead of them (measured per kernel family: the other choice costs either 1-4 %;
+            // a step or two later costs 9-25 %)
+            constexpr bool LATE_AHEAD = A_T && B_T;
+            if (LATE_AHEAD && late && st >= 1) issue(st + 1, buf_idx(st + 1));
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0, S0{});
-            if (late && st >= 1) issue(st + 1, buf_idx(st + 1));
+            if (!LATE_AHEAD && late && st >= 1) issue(st + 1, buf_idx(st + 1));
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1, S1{});
