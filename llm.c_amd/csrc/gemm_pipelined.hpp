@@ -93,6 +93,9 @@ constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 // one machine, both libraries loaded in one process and called in turn: NT bias kernels +2 to +7 % (fc 0.299 -> 0.315 ms,
 // fcproj 0.266 -> 0.285, qkv 0.206 -> 0.217), NT GELU +3 to +5 %, NN store within +-1 %, NN GELU backward +20 %. python llm.c_amd/build.py --variant rowwise -DLLMK_ROWWISE_LAST=1 builds it for
 // llm.c_amd/microbench.py --variant rowwise (2: also the GELU-backward kernels).
+#ifndef LLMK_DGELU_ASM
+#define LLMK_DGELU_ASM 1
+#endif
 #ifndef LLMK_ROWWISE_LAST
 #define LLMK_ROWWISE_LAST 0
 #endif
@@ -117,6 +120,10 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
+// Registers loaded by inline asm, whose completion the compiler does not track: after the wait for them they pass through
+// here, so that nothing that reads them can move above it
+template <typename V>
+__device__ __forceinline__ void tie4(V& a, V& b, V& c, V& d) { asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d)); }
 
 // Workgroup barrier WITHOUT the memory fence of __syncthreads(): the fence would wait for every outstanding
 // direct-to-LDS load (vmcnt(0)) and serialize the pipeline. Visibility of the K block that is about to be
@@ -473,6 +480,22 @@ gemm_pipelined_kernel(GemmArgs g) {
     // of little else; 1-2 % slower for the epilogues with activation math, so only that one takes this form)
     constexpr bool UNIFORM_GROUPS = EPI == EPI_DGELU_D;
     bool tile_inside = false;            // the tile whose epilogue is running (or about to) lies wholly inside the output
+    auto group_base = [&](const floatX* buf, int row0, int col0) -> const char* {      // the wave-uniform part of group_ptr
+        const size_t off = ((size_t)row0 * g.ldc + col0) * sizeof(floatX);
+        const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)off);
+        const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(off >> 32));
+        return reinterpret_cast<const char*>(buf) + (((size_t)hi << 32) | lo);
+    };
+    // The stored-derivative epilogue's loads, interior tiles: issued from inline asm and awaited by count, like the stage
+    // loads. Left to the compiler, every wait for them is a wait for (nearly) everything in flight: the compiler cannot see
+    // the hand-issued stage requests between them, and the epilogue's per-lane edge tests put each of its loads and stores
+    // behind a branch, which makes its own count of younger operations collapse to 0-2 - each 32-row block then waits for
+    // the previous block's stores to be acknowledged and for the next block's derivatives to arrive, four memory round
+    // trips per tile with the matrix cores idle. pre_young[b]: stage requests (units of CPW loads) issued behind the loads
+    // of block b (b = 0, 1; the later blocks' loads are issued inside the epilogue, where no stage is requested).
+    constexpr bool PRE_ASM = LLMK_DGELU_ASM && UNIFORM_GROUPS && LLMK_ROWWISE_LAST < 2 && LLMK_GEMM_ABL == 0;
+    constexpr int PRE_PB = PASSES * 4;   // derivative loads, and output stores, per 32-row block and wave
+    int pre_young[2] = {0, 0};
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
         if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
@@ -481,8 +504,14 @@ gemm_pipelined_kernel(GemmArgs g) {
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
-                    for (int t = 0; t < 4; t++)
-                        pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(group_ptr(g.aux, wm0 + i * 32 + t * 8, wn0 + pass * 64));
+                    for (int t = 0; t < 4; t++) {
+                        if constexpr (PRE_ASM) {
+                            asm volatile("global_load_dwordx4 %0, %1, %2" : "=v"(pre_act[i][pass][t])
+                                         : "v"(row_lane_off), "s"(group_base(g.aux, wm0 + i * 32 + t * 8, wn0 + pass * 64)));
+                        } else {
+                            pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(group_ptr(g.aux, wm0 + i * 32 + t * 8, wn0 + pass * 64));
+                        }
+                    }
                 return;
             }
 #pragma unroll
@@ -492,7 +521,13 @@ gemm_pipelined_kernel(GemmArgs g) {
                     const int row = t * 8 + (lane >> 3), ch = lane & 7;
                     const int m = wm0 + i * 32 + row;
                     const int n = wn0 + pass * 64 + ch * 8;
-                    if (m < g.M && n < g.N) pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(g.aux + (size_t)m * g.ldc + n);
+                    if (m < g.M && n < g.N) {
+                        if constexpr (PRE_ASM) {   // (no load of this kernel is left to the compiler's counting: it would await them all before each hand-issued one)
+                            asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(pre_act[i][pass][t]) : "v"(g.aux + (size_t)m * g.ldc + n));
+                        } else {
+                            pre_act[i][pass][t] = *reinterpret_cast<const u32x4*>(g.aux + (size_t)m * g.ldc + n);
+                        }
+                    }
                 }
             return;
         }
@@ -569,15 +604,36 @@ gemm_pipelined_kernel(GemmArgs g) {
     // writes the 4-column pieces it owns, then the wave reads the rows back 8 lanes to a row and stores
     // full 128-byte lines. e_m0, e_n0, e_split: the tile (they outlive the tile change, which renames the current one).
     int e_m0 = 0, e_n0 = 0, e_split = 0;
+    // the derivatives of block i have arrived (PRE_ASM, interior tile). Younger operations of the wave, in issue order: the
+    // stage requests counted in pre_young (blocks 0 and 1), the loads of the blocks requested after this one and the stores
+    // of the blocks that ran since. The registers are tied to the wait so that nothing that reads them moves above it.
+    auto await_pre = [&](auto ic) {
+        if constexpr (PRE_ASM) {
+            constexpr int i = decltype(ic)::value;
+            static_assert(PASSES == 1, "one pass per block");
+            constexpr int NEXT = i + 1 < TM ? PRE_PB : 0;         // the next block's loads: behind this block's, ahead of its wait
+            constexpr int BASE = i == 0 ? NEXT : PRE_PB + NEXT;   // ... and the previous block's stores
+            if (!tile_inside) wait_vmcnt<0>();                    // an edge tile: lanes outside load and store nothing, no count holds
+            else if (i >= 2 || pre_young[i < 2 ? i : 0] == 0) wait_vmcnt<BASE>();
+            else if (pre_young[i < 2 ? i : 0] == 1) wait_vmcnt<BASE + CPW>();
+            else wait_vmcnt<BASE + 2 * CPW>();
+            tie4(pre_act[i][0][0], pre_act[i][0][1], pre_act[i][0][2], pre_act[i][0][3]);
+        }
+    };
     auto epi_block = [&](auto ic) {
         constexpr int i = decltype(ic)::value;
         const int cur_m0 = e_m0, cur_n0 = e_n0, cur_split = e_split;
         char* strip = lds + STAGES * STAGE + wave * STRIP;
         const int wm0 = cur_m0 + wm * WTM, wn0 = cur_n0 + wn * WTN;
         constexpr int JP = F32OUT ? 1 : 2;                    // 32-column blocks per pass
-        const int wswz = (idx >> 1) & 7;
         (void)cur_split;
+        // (PRE_ASM: the lane's strip addresses are formed anew in every block. As loop invariants they were spilled, and a
+        // reload is a load the compiler awaits with vmcnt(0): the stage requests and derivative loads in flight with it)
+        int e_lane = lane;
+        if constexpr (PRE_ASM) asm volatile("" : "+v"(e_lane));
         {
+                const int lane = e_lane, idx = lane & 31, half = lane >> 5;
+                const int wswz = (idx >> 1) & 7;
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++) {
                     // phase 1: lane (row = idx, half) owns columns 8q + 4*half + 0..3 of each 32-column block
@@ -603,6 +659,7 @@ gemm_pipelined_kernel(GemmArgs g) {
                     }
                     __builtin_amdgcn_s_waitcnt(0xC07F);          // lgkmcnt(0): the strip is written
                     __builtin_amdgcn_wave_barrier();
+                    await_pre(ic);
                     // phase 2: 32 rows x 128 B, 8 lanes per row
 #pragma unroll
                     for (int t = 0; t < 4; t++) {
@@ -764,8 +821,9 @@ gemm_pipelined_kernel(GemmArgs g) {
                 voff_edge = edge;
                 par = 0;
                 issue(0, 0);
+                pre_young[0]++; pre_young[1]++;
             }
-            if (next_nkb > 1) issue(1, (1 + par) & 1);
+            if (next_nkb > 1) { issue(1, (1 + par) & 1); pre_young[0]++; pre_young[1]++; }
         };
         e_m0 = m0; e_n0 = n0; e_split = split;
         if constexpr (ROWWISE) {
@@ -836,12 +894,13 @@ gemm_pipelined_kernel(GemmArgs g) {
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0, S0{});
-            if (EARLY0 && !HAS_BIAS && late && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
+            pre_young[0] = pre_young[1] = 0;
+            if (EARLY0 && !HAS_BIAS && late && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; }
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1, S1{});
             bias_ready();                                         // two 16-wide steps after the request
-            if (EARLY0 && HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(nst - 2));
+            if (EARLY0 && HAS_BIAS && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; }
             read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0, S2{});
