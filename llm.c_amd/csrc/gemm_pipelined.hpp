@@ -477,8 +477,9 @@ gemm_pipelined_kernel(GemmArgs g) {
         return const_cast<char*>(reinterpret_cast<const char*>(buf)) + (((size_t)hi << 32) | lo) + row_lane_off;
     };
     // (measured: 4 % off the kernel whose epilogue only multiplies by a stored derivative, which is short of registers and
-    // of little else; 1-2 % slower for the epilogues with activation math, so only that one takes this form)
-    constexpr bool UNIFORM_GROUPS = EPI == EPI_DGELU_D;
+    // of little else; 1-2 % slower for the forward epilogues with activation math. The two backward GELU epilogues take
+    // this form: it is also what their hand-issued loads below address by)
+    constexpr bool UNIFORM_GROUPS = epi_gelu_bwd(EPI);
     bool tile_inside = false;            // the tile whose epilogue is running (or about to) lies wholly inside the output
     auto group_base = [&](const floatX* buf, int row0, int col0) -> const char* {      // the wave-uniform part of group_ptr
         const size_t off = ((size_t)row0 * g.ldc + col0) * sizeof(floatX);
@@ -486,8 +487,8 @@ gemm_pipelined_kernel(GemmArgs g) {
         const unsigned hi = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)(off >> 32));
         return reinterpret_cast<const char*>(buf) + (((size_t)hi << 32) | lo);
     };
-    // The stored-derivative epilogue's loads, interior tiles: issued from inline asm and awaited by count, like the stage
-    // loads. Left to the compiler, every wait for them is a wait for (nearly) everything in flight: the compiler cannot see
+    // The loads of the backward GELU epilogues (stored derivatives or pre-activations), interior tiles: issued from inline
+    // asm and awaited by count, like the stage loads. Left to the compiler, every wait for them is a wait for (nearly) everything in flight: the compiler cannot see
     // the hand-issued stage requests between them, and the epilogue's per-lane edge tests put each of its loads and stores
     // behind a branch, which makes its own count of younger operations collapse to 0-2 - each 32-row block then waits for
     // the previous block's stores to be acknowledged and for the next block's derivatives to arrive, four memory round
