@@ -96,6 +96,9 @@ constexpr int SK_MAX_ITEMS = 8;         // most short pieces one workgroup takes
 #ifndef LLMK_DGELU_ASM
 #define LLMK_DGELU_ASM 1
 #endif
+#ifndef LLMK_BIAS_ASM
+#define LLMK_BIAS_ASM 1
+#endif
 #ifndef LLMK_ROWWISE_LAST
 #define LLMK_ROWWISE_LAST 0
 #endif
@@ -552,14 +555,20 @@ gemm_pipelined_kernel(GemmArgs g) {
     // fp32 addition, as the epilogue's vector add gave it; that is TM x TN matrix instructions per tile while the matrix
     // cores would idle anyway, in place of an unpack and an add per element of the epilogue (64 vector instructions per
     // 32-row block), and two 2-byte loads per lane in place of eight 8-byte ones. Lanes past N, or a null bias, add zero:
-    // the epilogue has no bias code at all. The loads are ordinary loads, which the compiler awaits with vmcnt(0) - that
-    // also waits for every hand-issued tile load in flight - so they are placed in the one window in which this wave has
-    // none: from the start of the tile's last stage (the last-but-one stage ended with a wait for everything) until the
-    // wave requests the next tile's first stage, which these kernels do only after claiming the bias (bias_ready),
-    // half-way through the last stage.
+    // the epilogue has no bias code at all. The loads are requested at the start of the tile's last stage and claimed
+    // (bias_ready) half-way through it. As ordinary loads the compiler awaits them with vmcnt(0), which also waits for
+    // every hand-issued tile load in flight, so a kernel with such loads cannot request the next tile's first stage
+    // before it has claimed its bias (BIAS_LATE below); the product kernels issue and count them by hand (BIAS_ASM).
     constexpr bool HAS_BIAS = (EPI == EPI_BIAS || epi_gelu_fwd(EPI));
     unsigned biasw[HAS_BIAS ? TN : 1];   // bias of column j*32 + idx of the wave tile in the low 16 bits (lanes 0-31; 0 in lanes 32-63)
     bool bias_lane[HAS_BIAS ? TN : 1];
+    // BIAS_ASM: the two bias loads are issued from inline asm and awaited by count, so the next tile's first stage can be
+    // requested as early as in the kernels without a bias (the early waves a whole stage before this tile's last one);
+    // bias_young: a stage request of this wave sits behind them. BIAS_LATE (the row-wise variant and the ablation builds):
+    // ordinary loads, awaited by the compiler with vmcnt(0), and no stage request until they are claimed.
+    constexpr bool BIAS_ASM = HAS_BIAS && LLMK_BIAS_ASM && LLMK_ROWWISE_LAST == 0 && LLMK_GEMM_ABL == 0;
+    constexpr bool BIAS_LATE = HAS_BIAS && !BIAS_ASM;
+    bool bias_young = false;
     auto request_bias = [&](int n0) {
         if constexpr (HAS_BIAS) {
 #pragma unroll
@@ -569,13 +578,16 @@ gemm_pipelined_kernel(GemmArgs g) {
                 // unconditional, so that the value stays in the register it arrives in: lanes without a bias read the first
                 // bytes of A, which are there, and drop what they got when they claim it
                 const floatX* bp = bias_lane[j] ? g.bias + n : g.A;
-                biasw[j] = *reinterpret_cast<const unsigned short*>(bp);
+                if constexpr (BIAS_ASM) asm volatile("global_load_ushort %0, %1, off" : "=v"(biasw[j]) : "v"(bp));
+                else biasw[j] = *reinterpret_cast<const unsigned short*>(bp);
             }
+            bias_young = false;
             asm volatile("" ::: "memory");                        // the loads stay here: nothing below may pull them down to their use
         }
     };
     auto bias_ready = [&]() {
         if constexpr (HAS_BIAS) {
+            if constexpr (BIAS_ASM) { if (bias_young) wait_vmcnt<CPW>(); else wait_vmcnt<0>(); }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 asm volatile("" : "+v"(biasw[j]));
@@ -799,7 +811,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             barrier_no_fence();                              // ... and for everyone; the buffer of stage st is free
             if (!late) {
                 if (st + 2 < nst) issue(st + 2, buf_idx(st));
-                else if (EARLY0 && !HAS_BIAS && early0) issue_from(tile_base_n, 0, buf_idx(st));
+                else if (EARLY0 && !BIAS_LATE && early0) issue_from(tile_base_n, 0, buf_idx(st));
             }
             read_frags(buf_of(st + 1), S0{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
@@ -896,12 +908,12 @@ gemm_pipelined_kernel(GemmArgs g) {
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0, S0{});
             pre_young[0] = pre_young[1] = 0;
-            if (EARLY0 && !HAS_BIAS && late && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; }
+            if (EARLY0 && !BIAS_LATE && late && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; bias_young = true; }
             read_frags(cur, S2{}, fa0, fb0);
             await_frags(fa1, fb1, Younger{});
             mma(fa1, fb1, S1{});
             bias_ready();                                         // two 16-wide steps after the request
-            if (EARLY0 && HAS_BIAS && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; }
+            if (EARLY0 && BIAS_LATE && early0) { issue_from(tile_base_n, 0, buf_idx(nst - 2)); pre_young[0]++; }
             read_frags(cur, S3{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});
             mma(fa0, fb0, S2{});
