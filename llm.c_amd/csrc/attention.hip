@@ -733,8 +733,10 @@ fa_backward_dkdv_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ do
 __global__ void __launch_bounds__(256)
 fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ dout, const floatX* __restrict__ qkv,
                         const float* __restrict__ stats, const float* __restrict__ Dsum, int T, int NH, int nk) {
-    __shared__ __attribute__((aligned(1024))) char sQ[2][SW_TILE];
-    __shared__ __attribute__((aligned(1024))) char sdO[2][SW_TILE];
+    // Q tiles in sT[0..1], dO tiles in sT[2..3]. One array, aligned to twice the tile pair: the buffer in use is bit 13 of an
+    // LDS address, and the dO tile of a buffer is a constant 2 * SW_TILE behind its Q tile.
+    __shared__ __attribute__((aligned(4 * SW_TILE))) char sT[4][SW_TILE];
+    static_assert(SW_TILE == 0x2000, "the buffer toggle below is an XOR with the tile size");
     extern __shared__ __attribute__((aligned(16))) float sStat[];   // [2][T]: log-sum-exp (in log2 units) and -rowsum(dO*O) of every query of this head
     float* sLall = sStat;
     float* sDall = sStat + T;
@@ -765,14 +767,38 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
     {
         const int q_first = (kt_first * 128) / 64;
         if (q_first < q_end) {
-            fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sQ[0]), uwave);
-            fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sdO[0]), uwave);
+            fa_tile_request(laq, base + (size_t)(64 * q_first) * C3, fa_lds_addr(sT[0]), uwave);
+            fa_tile_request(lado, dobase + (size_t)(64 * q_first) * C, fa_lds_addr(sT[2]), uwave);
         }
         // the per-query statistics of the head go to LDS once (the first tile's queries include the second's): no global
         // loads besides the tiles inside the loops
         for (int q = 64 * q_first + tid; q < T; q += 256) { sLall[q] = lbase[q] * LOG2E; sDall[q] = -dbase[q]; }    // negated: see below
     }
     int buf = 0;
+    // LDS addresses of this lane's operand pieces in the Q tile of the buffer in use, one register each: the four K steps
+    // of a fragment along rows, and the two 8-byte pieces of a transposing read for the two column halves. Everything
+    // else about a read (the 32-query block, the 16-query step, the dO tile) is an immediate offset, and the change of
+    // buffer is one XOR per register and iteration: no address arithmetic at the reads themselves (it was a vector add
+    // per read, a quarter of the loop's vector instructions).
+    unsigned ar[4], ac[4];
+    {
+        const unsigned t0 = fa_lds_addr(sT[0]);
+#pragma unroll
+        for (int s = 0; s < 4; s++) ar[s] = t0 + (laq.rowb ^ (unsigned)(s << 5));
+        ac[0] = t0 + laq.colb0; ac[1] = t0 + laq.colb1; ac[2] = t0 + (laq.colb0 ^ 64u); ac[3] = t0 + (laq.colb1 ^ 64u);
+    }
+    typedef const __attribute__((address_space(3))) bf16x8* lds_frag_ptr;
+    typedef s16x4 __attribute__((address_space(3))) * lds_tr_ptr;
+    auto rows_frag = [&](bool of_do, int qb, int s) -> bf16x8 {
+        return *reinterpret_cast<lds_frag_ptr>((size_t)(ar[s] + (unsigned)(32 * qb * 128 + (of_do ? 2 * SW_TILE : 0))));
+    };
+    auto cols_frag = [&](bool of_do, int kbase, int d) -> bf16x8 {
+        const unsigned off = (unsigned)(kbase * 128 + (of_do ? 2 * SW_TILE : 0));
+        union { struct { s16x4 a, b; } s; bf16x8 v; } u;
+        u.s.a = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(size_t)(ac[2 * d] + off));
+        u.s.b = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr)(size_t)(ac[2 * d + 1] + off));
+        return u.v;
+    };
 
     for (int phase = 0; phase < nphase; phase++) {
         const int kt = phase == 0 ? kt_first : kt_second;
@@ -800,17 +826,18 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
         fa_tiles_landed();                               // the wave's own rows (and, first time, the first tiles and the statistics)
         if (phase == 0) __syncthreads();
 
+        // this lane's four statistics of a 16-query group: one address register per table, advanced by a tile per iteration
+        unsigned stat_l = fa_lds_addr(sLall + 64 * q_first) + (unsigned)(lane >> 5) * 16u;
+        unsigned stat_d = fa_lds_addr(sDall + 64 * q_first) + (unsigned)(lane >> 5) * 16u;
         for (int qi = q_first; qi < q_end; qi++) {
-            const unsigned tq = fa_lds_addr(sQ[buf]), tdo = fa_lds_addr(sdO[buf]);
             buf ^= 1;
-            const unsigned stat_l = fa_lds_addr(sLall + 64 * qi), stat_d = fa_lds_addr(sDall + 64 * qi);
             if (qi + 1 < q_end) {
-                fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sQ[buf]), uwave);
-                fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sdO[buf]), uwave);
+                fa_tile_request(laq, base + (size_t)(64 * (qi + 1)) * C3, fa_lds_addr(sT[buf]), uwave);
+                fa_tile_request(lado, dobase + (size_t)(64 * (qi + 1)) * C, fa_lds_addr(sT[2 + buf]), uwave);
             } else if (phase + 1 < nphase) {             // the second tile's first queries
                 const int qn = (kt_second * 128) / 64;
-                fa_tile_request(laq, base + (size_t)(64 * qn) * C3, fa_lds_addr(sQ[buf]), uwave);
-                fa_tile_request(lado, dobase + (size_t)(64 * qn) * C, fa_lds_addr(sdO[buf]), uwave);
+                fa_tile_request(laq, base + (size_t)(64 * qn) * C3, fa_lds_addr(sT[buf]), uwave);
+                fa_tile_request(lado, dobase + (size_t)(64 * qn) * C, fa_lds_addr(sT[2 + buf]), uwave);
             }
 #pragma unroll
             for (int qb = 0; qb < 2; qb++) {
@@ -822,7 +849,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 for (int r = 0; r < 16; r++) sacc[r] = 0.f;
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8 + half * 4) * 4);
+                    const f32x4 d4 = fa_lds_f32x4(stat_d + (32 * qb + g * 8) * 4);
 #pragma unroll
                     for (int e = 0; e < 4; e++) pacc[4 * g + e] = d4[e];
                 }
@@ -833,13 +860,12 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 constexpr int LAG = 4;                           // steps by which the dP chain runs behind the S chain
 #pragma unroll
                 for (int s = 0; s < 4 + LAG; s++) {
-                    if (s < 4) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tq, laq, 32 * qb, s), kf[s], sacc, 0, 0, 0);
-                    if (s >= LAG) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows(tdo, laq, 32 * qb, s - LAG), vf[s - LAG], pacc, 0, 0, 0);
+                    if (s < 4) sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag(false, qb, s), kf[s], sacc, 0, 0, 0);
+                    if (s >= LAG) pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(rows_frag(true, qb, s - LAG), vf[s - LAG], pacc, 0, 0, 0);
                 }
 #pragma unroll
                 for (int g = 0; g < 4; g++) {
-                    const int rr = 32 * qb + g * 8 + half * 4;
-                    const f32x4 l4 = fa_lds_f32x4(stat_l + rr * 4);
+                    const f32x4 l4 = fa_lds_f32x4(stat_l + (32 * qb + g * 8) * 4);
 #pragma unroll
                     for (int e = 0; e < 4; e++) sacc[4 * g + e] = fast_exp2(fmaf(sacc[4 * g + e], c, -l4[e]));
                 }
@@ -860,16 +886,19 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                     const bf16x8 pf = pack_acc(sacc, s2);
 #pragma unroll
                     for (int d = 0; d < 2; d++)
-                        dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tdo, laq, 32 * qb + 16 * s2, 32 * d), pf, dv[d], 0, 0, 0);
+                        dv[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag(true, 32 * qb + 16 * s2, d), pf, dv[d], 0, 0, 0);
                 }
 #pragma unroll
                 for (int s2 = 0; s2 < 2; s2++) {
                     const bf16x8 dsf = pack_acc(pacc, s2);
 #pragma unroll
                     for (int d = 0; d < 2; d++)
-                        dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols(tq, laq, 32 * qb + 16 * s2, 32 * d), dsf, dk[d], 0, 0, 0);
+                        dk[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(cols_frag(false, 32 * qb + 16 * s2, d), dsf, dk[d], 0, 0, 0);
                 }
             }
+#pragma unroll
+            for (int s = 0; s < 4; s++) { ar[s] ^= (unsigned)SW_TILE; ac[s] ^= (unsigned)SW_TILE; }    // the other buffer
+            stat_l += 256u; stat_d += 256u;
             fa_tiles_landed();
             __syncthreads();
         }
