@@ -187,8 +187,20 @@ __device__ __forceinline__ bf16x8 fa_frag_rows(unsigned tile, const FaLane& a, i
 __device__ __forceinline__ unsigned fa_fresh(unsigned v) { asm volatile("" : "+v"(v)); return v; }
 // The same reads for a kernel short of registers: the swizzled address of each step is formed at the read (one
 // xor-add) rather than held for the life of the kernel.
-__device__ __forceinline__ bf16x8 fa_frag_rows_lean(unsigned tile, const FaLane& a, int row0, int s) {
-    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)((fa_fresh(a.rowb) ^ (unsigned)(s << 5)) + (tile + row0 * 128)));
+// (lane ^ X) + tile as ONE vector instruction issued where it is written: stated in asm, the compiler neither hoists the
+// four (eight) variants of an address into registers of their own nor copies the lane part first to protect it. X has to
+// be an inline constant (0, 32, 64); 96 takes a xor and an add. `tile` is wave-uniform (a scalar register).
+template <int X>
+__device__ __forceinline__ unsigned fa_xad(unsigned lane_part, unsigned tile) {
+    unsigned r;
+    if constexpr (X == 0) asm volatile("v_add_u32 %0, %2, %1" : "=v"(r) : "v"(lane_part), "s"(tile));
+    else if constexpr (X <= 64) asm volatile("v_xad_u32 %0, %1, %2, %3" : "=v"(r) : "v"(lane_part), "n"(X), "s"(tile));
+    else asm volatile("v_xor_b32 %0, %2, %1\n\tv_add_u32 %0, %3, %0" : "=&v"(r) : "v"(lane_part), "n"(X), "s"(tile));
+    return r;
+}
+template <int S>
+__device__ __forceinline__ bf16x8 fa_frag_rows_lean(unsigned tile, const FaLane& a, int row0) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)(fa_xad<(S << 5)>(a.rowb, tile) + (unsigned)(row0 * 128)));
 }
 __device__ __forceinline__ f32x4 fa_lds_f32x4(unsigned addr) {
     return *reinterpret_cast<const __attribute__((address_space(3))) f32x4*>((size_t)addr);
@@ -204,11 +216,13 @@ __device__ __forceinline__ bf16x8 fa_frag_cols(unsigned tile, const FaLane& a, i
     return u.v;
 }
 
-__device__ __forceinline__ bf16x8 fa_frag_cols_lean(unsigned tile, const FaLane& a, int kbase, int col0) {
+template <int COL0>
+__device__ __forceinline__ bf16x8 fa_frag_cols_lean(unsigned tile, const FaLane& a, int kbase) {
     typedef s16x4 __attribute__((address_space(3))) * lds_ptr;
-    const unsigned x = col0 ? 64u : 0u, t = tile + kbase * 128;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)((fa_fresh(a.colb0) ^ x) + t));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)((fa_fresh(a.colb1) ^ x) + t));
+    constexpr int X = COL0 ? 64 : 0;
+    const unsigned off = (unsigned)(kbase * 128);
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(fa_xad<X>(a.colb0, tile) + off));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(size_t)(fa_xad<X>(a.colb1, tile) + off));
     union { struct { s16x4 a, b; } s; bf16x8 v; } u;
     u.s.a = lo; u.s.b = hi;
     return u.v;
@@ -898,7 +912,9 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
             }
 #pragma unroll
             for (int s = 0; s < 4; s++) { ar[s] ^= (unsigned)SW_TILE; ac[s] ^= (unsigned)SW_TILE; }    // the other buffer
-            stat_l += 256u; stat_d += 256u;
+            // (in asm: as a plain addition the compiler re-bases the reads on the advanced value, with negative offsets that
+            // a read cannot encode, and is back to an add per read)
+            asm volatile("v_add_u32 %0, 0x100, %0\n\tv_add_u32 %1, 0x100, %1" : "+v"(stat_l), "+v"(stat_d));
             fa_tiles_landed();
             __syncthreads();
         }
@@ -1108,12 +1124,14 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
                 f32x16 sacc, pacc;
 #pragma unroll
                 for (int r = 0; r < 16; r++) { sacc[r] = 0.f; pacc[r] = 0.f; }
-#pragma unroll
-                for (int s = 0; s < 4; s++)
-                    sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean(tk, la, 32 * kb, s), qf[s], sacc, 0, 0, 0);
-#pragma unroll
-                for (int s = 0; s < 4; s++)
-                    pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean(tv, la, 32 * kb, s), dof[s], pacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<0>(tk, la, 32 * kb), qf[0], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<1>(tk, la, 32 * kb), qf[1], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<2>(tk, la, 32 * kb), qf[2], sacc, 0, 0, 0);
+                sacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<3>(tk, la, 32 * kb), qf[3], sacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<0>(tv, la, 32 * kb), dof[0], pacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<1>(tv, la, 32 * kb), dof[1], pacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<2>(tv, la, 32 * kb), dof[2], pacc, 0, 0, 0);
+                pacc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_rows_lean<3>(tv, la, 32 * kb), dof[3], pacc, 0, 0, 0);
 #pragma unroll
                 for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
                 if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
@@ -1129,9 +1147,8 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
 #pragma unroll
                 for (int s2 = 0; s2 < 2; s2++) {
                     const bf16x8 dsf = pack_acc(pacc, s2);
-#pragma unroll
-                    for (int d = 0; d < 2; d++)
-                        dq[d] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols_lean(tk, la, 32 * kb + 16 * s2, 32 * d), dsf, dq[d], 0, 0, 0);
+                    dq[0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols_lean<0>(tk, la, 32 * kb + 16 * s2), dsf, dq[0], 0, 0, 0);
+                    dq[1] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa_frag_cols_lean<32>(tk, la, 32 * kb + 16 * s2), dsf, dq[1], 0, 0, 0);
                 }
             }
             fa_tiles_landed();
