@@ -249,12 +249,15 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
         const size_t base = (size_t)row * C;
 #pragma unroll
         for (int i = 0; i < NV; i++) {
-            int v = lane + i * 64;
-            if (v < nvec) {
-                g[i] = ld_vec_nt(dout + base + (size_t)v * VN);
-                x[i] = ld_vec_nt(inp + base + (size_t)v * VN);
-                di[i] = ld_vec_nt(dinp + base + (size_t)v * VN);
-            }
+            // Every lane loads, the lanes past the row's end a copy of its last vector (NV = ceil(nvec / 64), so only the
+            // last slot has such lanes; what they hold is never added to a sum nor stored). With the loads under a
+            // per-lane test each sits behind a branch that may skip it, the compiler's count of loads certainly younger
+            // than the ones it waits for drops to zero, and the wait for the current row also waits for the row
+            // requested ahead: one row in flight instead of two.
+            const int v = i == NV - 1 ? min(lane + i * 64, nvec - 1) : lane + i * 64;
+            g[i] = ld_vec_nt(dout + base + (size_t)v * VN);
+            x[i] = ld_vec_nt(inp + base + (size_t)v * VN);
+            di[i] = ld_vec_nt(dinp + base + (size_t)v * VN);
         }
     };
     auto process_row = [&](int row, float m, float r, vecX (&g)[NV], vecX (&x)[NV], vecX (&di)[NV]) {
@@ -305,19 +308,26 @@ ln_backward_kernel(floatX* __restrict__ dinp, float* __restrict__ partial, const
             process_row(row, mean[row], rstd[row], g0, x0, d0);
         }
     } else {
+        // The row index is kept wave-uniform and the row requested ahead is requested unconditionally (past the end: the
+        // last row again, never processed): loop control is scalar branches around straight-line loads, which is what
+        // the compiler needs to count the loads behind the ones it waits for. With the request under a per-lane test of
+        // the row index, every wait for the current row was a wait for everything in flight.
         vecX g0[NV], x0[NV], d0[NV], g1[NV], x1[NV], d1[NV];
-        int row = wave;
+        int row = __builtin_amdgcn_readfirstlane(wave);
         float m0 = 0.f, r0 = 0.f, m1 = 0.f, r1 = 0.f;
-        if (row < N) { load_row(row, g0, x0, d0); m0 = mean[row]; r0 = rstd[row]; }
-        while (row < N) {
-            const int row1 = row + nwaves;
-            if (row1 < N) { load_row(row1, g1, x1, d1); m1 = mean[row1]; r1 = rstd[row1]; }
-            process_row(row, m0, r0, g0, x0, d0);
-            if (row1 >= N) break;
-            const int row2 = row1 + nwaves;
-            if (row2 < N) { load_row(row2, g0, x0, d0); m0 = mean[row2]; r0 = rstd[row2]; }
-            process_row(row1, m1, r1, g1, x1, d1);
-            row = row2;
+        if (row < N) {
+            load_row(row, g0, x0, d0); m0 = mean[row]; r0 = rstd[row];
+            while (true) {
+                const int row1 = row + nwaves, row1c = min(row1, N - 1);
+                load_row(row1c, g1, x1, d1); m1 = mean[row1c]; r1 = rstd[row1c];
+                process_row(row, m0, r0, g0, x0, d0);
+                if (row1 >= N) break;
+                const int row2 = row1 + nwaves, row2c = min(row2, N - 1);
+                load_row(row2c, g0, x0, d0); m0 = mean[row2c]; r0 = rstd[row2c];
+                process_row(row1, m1, r1, g1, x1, d1);
+                if (row2 >= N) break;
+                row = row2;
+            }
         }
     }
 
