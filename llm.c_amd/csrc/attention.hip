@@ -20,6 +20,7 @@
 // parity runs against the CPU reference at small sizes.
 #include "common.hpp"
 #include <type_traits>
+#include <utility>
 #include "../../include/llmk.h"
 
 namespace {
@@ -86,6 +87,36 @@ __device__ __forceinline__ float fa_max_with_other_half(float v) {
 }
 // row index (within a 32-row block) of accumulator register r for this lane
 __device__ __forceinline__ int acc_row(int r, int lane) { return (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3); }
+
+// The causal mask of a 32 x 32 block on the diagonal (its first row and its first column are the same position; the
+// direct-to-LDS kernels meet no other kind, all their blocks start at multiples of 32). Register r of lane l is row
+// acc_row(r, l) against column l % 32, so WHICH LANES are masked in register r is a constant of r: a 64-bit lane mask
+// that lives in scalar registers, and one select per element - where the per-lane form took an add, a compare and a
+// select each, with wait states between them, a tenth of the forward loop's vector instructions at T = 1024.
+// ROW_GT: rows past the column are masked (rows are keys: forward, dQ); else rows before it (rows are queries: dK/dV).
+template <int R, bool ROW_GT>
+constexpr unsigned long long fa_diag_lanes() {
+    unsigned long long m = 0;
+    for (int l = 0; l < 64; l++) {
+        const int row = (R >> 2) * 8 + (l >> 5) * 4 + (R & 3), col = l & 31;
+        if (ROW_GT ? row > col : row < col) m |= 1ull << l;
+    }
+    return m;
+}
+template <int R, bool ROW_GT>
+__device__ __forceinline__ float fa_mask_one(float x, float fill) {
+    // (the builtin, not the instruction in asm: x comes straight out of an MFMA, and the wait states between a matrix
+    // instruction and a vector instruction that reads its result are the compiler's to insert - it does not look into asm)
+    return __builtin_amdgcn_inverse_ballot_w64(fa_diag_lanes<R, ROW_GT>()) ? fill : x;
+}
+template <bool ROW_GT, int... R>
+__device__ __forceinline__ void fa_mask_diag_seq(f32x16& a, float fill, std::integer_sequence<int, R...>) {
+    ((a[R] = fa_mask_one<R, ROW_GT>(a[R], fill)), ...);
+}
+template <bool ROW_GT>
+__device__ __forceinline__ void fa_mask_diag(f32x16& a, float fill) {
+    fa_mask_diag_seq<ROW_GT>(a, fill, std::make_integer_sequence<int, 16>{});
+}
 
 // cooperative 64x64 bf16 tile copy global -> registers (2 x 16 B per thread, 256 threads)
 struct TileRegs { u32x4 v[2]; };
@@ -508,14 +539,15 @@ fa_forward_dma_kernel(floatX* __restrict__ out, float* __restrict__ stats, const
                 }
                 if (64 * j + 63 > qw0) {                      // diagonal tile: some (key, query) pairs are masked (wave-uniform test)
                     asm volatile("" ::: "memory");            // keep this a branch: off the diagonal the selects are pure overhead
-                    // key 64j + 32kb + acc_row(r) against query qw0 + idx: the lane's share of both sides is one small number
-                    const int ln = fresh_lane(lane);
-                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = qw0 - 64 * j;
+                    // qw0 - 64 j is 0 (the first 32 keys are the wave's diagonal block, the other 32 all in the future) or 32
+                    // (the first 32 all visible, the other 32 the diagonal block)
+                    if (qw0 == 64 * j) {
+                        fa_mask_diag<true>(sacc[0], -INFINITY);
 #pragma unroll
-                    for (int kb = 0; kb < 2; kb++)
-#pragma unroll
-                        for (int r = 0; r < 16; r++)
-                            if (32 * kb + (r >> 2) * 8 + (r & 3) + dl > lim) sacc[kb][r] = -INFINITY;
+                        for (int r = 0; r < 16; r++) sacc[1][r] = -INFINITY;
+                    } else {
+                        fa_mask_diag<true>(sacc[1], -INFINITY);
+                    }
                 }
                 float mx = fmaxf(sacc[0][0], sacc[1][0]);
 #pragma unroll
@@ -885,12 +917,7 @@ fa_backward_dkdv_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict_
                 }
                 if (q0 < kw0 + 31) {                             // diagonal block (wave-uniform test; T % 64 == 0: no rows past the end)
                     asm volatile("" ::: "memory");                // keep this a branch: off the diagonal the selects are pure overhead
-                    // query q0 + acc_row(r) against key kw0 + idx: the lane's share of both sides is one small number
-                    const int ln = fresh_lane(lane);
-                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = kw0 - q0;
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        if ((r >> 2) * 8 + (r & 3) + dl < lim) sacc[r] = 0.f;
+                    fa_mask_diag<false>(sacc, 0.f);               // q0 == kw0: query q0 + acc_row(r) against key kw0 + idx
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * pacc[r];
@@ -1136,11 +1163,7 @@ fa_backward_dq_dma_kernel(floatX* __restrict__ dqkv, const floatX* __restrict__ 
                 for (int r = 0; r < 16; r++) sacc[r] = fast_exp2(fmaf(sacc[r], c, -lse2));
                 if (k0 + 31 > qw0) {                              // diagonal block (wave-uniform test)
                     asm volatile("" ::: "memory");                // keep this a branch: off the diagonal the selects are pure overhead
-                    const int ln = fresh_lane(lane);
-                    const int dl = ((ln >> 5) << 2) - (ln & 31), lim = qw0 - k0;      // key k0 + acc_row(r) against query qw0 + idx
-#pragma unroll
-                    for (int r = 0; r < 16; r++)
-                        if ((r >> 2) * 8 + (r & 3) + dl > lim) sacc[r] = 0.f;
+                    fa_mask_diag<true>(sacc, 0.f);                // k0 == qw0: key k0 + acc_row(r) against query qw0 + idx
                 }
 #pragma unroll
                 for (int r = 0; r < 16; r++) pacc[r] = sacc[r] * (pacc[r] - dsum);
