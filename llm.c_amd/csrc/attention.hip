@@ -213,9 +213,6 @@ __device__ __forceinline__ unsigned fa_lds_addr(const void* p) {
 __device__ __forceinline__ bf16x8 fa_frag_rows(unsigned tile, const FaLane& a, int row0, int s) {
     return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((size_t)(tile + row0 * 128 + (a.rowb ^ (unsigned)(s << 5))));
 }
-// A value the compiler must take as new at this point: what is derived from it is computed here, next to its use,
-// instead of once before the loop and kept in a register of its own for the whole kernel.
-__device__ __forceinline__ unsigned fa_fresh(unsigned v) { asm volatile("" : "+v"(v)); return v; }
 // The same reads for a kernel short of registers: the swizzled address of each step is formed at the read (one
 // xor-add) rather than held for the life of the kernel.
 // (lane ^ X) + tile as ONE vector instruction issued where it is written: stated in asm, the compiler neither hoists the
