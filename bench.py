@@ -59,7 +59,7 @@ def measured_traffic(family):
 
 
 # kernel families timed by the library -> roofline that bounds them
-MFMA_BOUND = {"gemm_nt", "gemm_nt_gelu", "gemm_nn", "gemm_nn_dgelu", "gemm_tn", "gemm_tn_splitk",
+MFMA_BOUND = {"gemm_nt", "gemm_nt_gelu", "gemm_nt_res", "gemm_nn", "gemm_nn_dgelu", "gemm_tn", "gemm_tn_splitk",
               "attention_forward", "attention_backward_dkdv", "attention_backward_dq"}
 
 

@@ -138,6 +138,14 @@ size_t llmk_layernorm_backward_scratch_floats(int C);
 void llmk_matmul_forward(void* out, const void* inp, const void* weight, const void* bias, int B, int T, int C,
                          int OC, void* stream, void* pre_gelu, int gelu_fusion);
 
+/* The projection and the residual add that follows it in one launch: out = round(round(inp . weight^T + bias) + residual),
+ * both roundings to the storage type as llmk_matmul_forward followed by the add of llmk_fused_residual_forward5
+ * (llmc/layernorm.cuh:467, its residual = inp1 + inp2) give them, so the bits are the same. It has no counterpart in the
+ * reference (which runs matmul_forward_cublaslt and fused_residual_forward5, train_gpt2.cu:713-727); a LayerNorm of out
+ * (llmk_layernorm_forward) then takes the place of the fused kernel. out must not be residual or inp. */
+void llmk_matmul_forward_residual(void* out, const void* inp, const void* weight, const void* bias, const void* residual,
+                                  int B, int T, int C, int OC, void* stream);
+
 /* matmul_backward, llmc/matmul.cuh:244.
  *   dbias[OC]   += column sums of dout          (skipped when dbias == NULL)
  *   dinp[B*T,C]  = dout . weight                 (then *= gelu'(pre_gelu) when pre_gelu != NULL;

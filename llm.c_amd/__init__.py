@@ -63,6 +63,7 @@ KERNEL_ABI = {
     "llmk_layernorm_backward": (None, [vp, vp, vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, vp]),
     "llmk_layernorm_backward_scratch_floats": (sz, [i32]),
     "llmk_matmul_forward": (None, [vp, vp, vp, vp, i32, i32, i32, i32, vp, vp, i32]),
+    "llmk_matmul_forward_residual": (None, [vp, vp, vp, vp, vp, i32, i32, i32, i32, vp]),
     "llmk_matmul_backward": (None, [vp, vp, vp, vp, vp, vp, vp, i32, i32, i32, i32, vp, vp, i32]),
     "llmk_matmul_backward_bias_scratch_floats": (sz, [i32]),
     "llmk_gelu_backward_bias": (None, [vp, vp, vp, vp, i32, i32, i32, vp]),

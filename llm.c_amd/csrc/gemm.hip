@@ -774,6 +774,36 @@ size_t llmk_matmul_backward_workspace_bytes(int B, int T, int C, int OC) {
     return ((size_t)OC * C + (size_t)OC * 4) * pieces * sizeof(float);     // partial products + the bias gradient's row sums
 }
 
+// out = bf16(bf16(inp . weight^T + bias) + residual): the projection and the residual stream's add in one launch, with
+// both roundings of the two-kernel form (llmk_matmul_forward, then llmk_residual_forward or llmk_fused_residual_forward5's
+// add), so the bits are the same. out may be the residual buffer's successor or any other buffer; not inp.
+void llmk_matmul_forward_residual(void* out, const void* inp, const void* weight, const void* bias, const void* residual,
+                                  int B, int T, int C, int OC, void* stream) {
+    if (llmk::failed()) return;
+    const int M = B * T;
+    LLMK_REQUIRE(C % K_ALIGN == 0, "matmul_forward_residual: C=%d must be a multiple of %d", C, K_ALIGN);
+    LLMK_REQUIRE(aligned16(inp) && aligned16(weight), "matmul_forward_residual: operands must be 16-byte aligned");
+    if (M == 0 || OC == 0) return;
+    hipStream_t st = (hipStream_t)stream;
+#if !defined(LLMK_FP32)
+    GemmArgs g{};
+    g.A = (const floatX*)inp; g.B = (const floatX*)weight; g.M = M; g.N = OC; g.K = C;
+    g.lda = C; g.ldb = C; g.ldc = OC; g.bias = (const floatX*)bias; g.k_per_split = CEIL_DIV(C, K_STEP) * K_STEP;
+    g.C = (floatX*)out; g.aux = (floatX*)residual;
+    const bool big = (size_t)CEIL_DIV(M, BIG_TILE) * CEIL_DIV(OC, BIG_TILE) >= (size_t)llmk::device_info().num_cu;
+    if (big && out != residual && aligned16(residual) && aligned16(out) && pipelined_ok(g)) {
+        llmk::ProfScope prof("gemm_nt_res", 2.0 * M * (double)OC * C, ((double)M * C + (double)OC * C + 2.0 * M * OC) * sizeof(floatX), st);
+        launch_pipelined_cfg<256, 256, 2, 4, false, false, EPI_BIAS_RES>(g, 1, st);
+        return;
+    }
+#endif
+    // shapes the fused epilogue does not take: the two kernels (out first holds the projection, then the sum; the add reads
+    // and writes element by element, so in place is fine)
+    LLMK_REQUIRE(out != residual, "matmul_forward_residual: out must not be the residual buffer");
+    llmk_matmul_forward(out, inp, weight, bias, B, T, C, OC, stream, nullptr, 1);
+    llmk_residual_forward(out, residual, out, M * OC, stream);
+}
+
 void llmk_matmul_backward(void* dinp, void* dweight, void* dbias, const void* dout, const void* inp,
                           const void* weight, float* dbias_buffer, int B, int T, int C, int OC, void* stream,
                           const void* pre_gelu, int gelu_fusion) {

@@ -47,10 +47,14 @@ typedef __attribute__((ext_vector_type(4))) unsigned int u32x4;
 // EPI_BIAS_GELU_D / EPI_DGELU_D (gelu_fusion 3): the forward epilogue leaves gelu'(pre-activation) in the second output
 // instead of the pre-activation, and the backward epilogue multiplies by that stored value: the exponential, the
 // reciprocal and nine of the thirteen vector operations per element move out of the backward epilogue, four into the forward one.
+// EPI_BIAS_RES: C = bf16(bf16(acc + bias) + aux), the residual stream's add taken into the projection that feeds it
+// (both roundings of the two-kernel form: the GEMM's output rounded to bf16, then the sum).
 enum Epi { EPI_BIAS = 0, EPI_BIAS_GELU = 1, EPI_STORE = 2, EPI_DGELU = 3, EPI_ACCUM = 4, EPI_PARTIAL = 5, EPI_PARTIAL_ROWSUM = 6,
-           EPI_BIAS_GELU_D = 7, EPI_DGELU_D = 8 };
+           EPI_BIAS_GELU_D = 7, EPI_DGELU_D = 8, EPI_BIAS_RES = 9 };
 constexpr bool epi_gelu_fwd(int e) { return e == EPI_BIAS_GELU || e == EPI_BIAS_GELU_D; }
 constexpr bool epi_gelu_bwd(int e) { return e == EPI_DGELU || e == EPI_DGELU_D; }
+// epilogues that read a tensor of the output's shape (g.aux) with the lanes' store pattern
+constexpr bool epi_reads_aux(int e) { return epi_gelu_bwd(e) || e == EPI_BIAS_RES; }
 
 struct GemmArgs {
     const floatX* A;
@@ -465,10 +469,10 @@ gemm_pipelined_kernel(GemmArgs g) {
     // last K blocks of the tile are still being multiplied: the addresses are the ones the epilogue will store to.
     constexpr bool F32OUT = (IS_PARTIAL || EPI == EPI_ACCUM);   // staged in fp32 so that C += acc rounds once
     constexpr int PASSES = F32OUT ? TN : TN / 2;          // a strip row is 128 B: 64 bf16 columns or 32 fp32 columns
-    constexpr bool EPI_READS = (EPI == EPI_ACCUM || epi_gelu_bwd(EPI));
+    constexpr bool EPI_READS = (EPI == EPI_ACCUM || epi_reads_aux(EPI));
     bf16x4 pre_old[EPI == EPI_ACCUM ? TM : 1][EPI == EPI_ACCUM ? PASSES : 1][2][2];
     // GELU backward: the pre-activation values of the 16 bytes each lane stores per (block, pass, quarter), as it stores them
-    u32x4 pre_act[epi_gelu_bwd(EPI) ? TM : 1][epi_gelu_bwd(EPI) ? PASSES : 1][4];
+    u32x4 pre_act[epi_reads_aux(EPI) ? TM : 1][epi_reads_aux(EPI) ? PASSES : 1][4];
     // Row groups of a tile that lies wholly inside the output (no lane tests its row or column): 8 rows x 128 B, lane
     // (row = lane / 8, chunk = lane % 8) at a wave-uniform base (scalar registers) plus one per-lane byte offset that is the
     // same for every group of every tile. The general form costs each load and store a 64-bit address of its own.
@@ -482,7 +486,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     // (measured: 4 % off the kernel whose epilogue only multiplies by a stored derivative, which is short of registers and
     // of little else; 1-2 % slower for the forward epilogues with activation math. The two backward GELU epilogues take
     // this form: it is also what their hand-issued loads below address by)
-    constexpr bool UNIFORM_GROUPS = epi_gelu_bwd(EPI);
+    constexpr bool UNIFORM_GROUPS = epi_reads_aux(EPI);
     bool tile_inside = false;            // the tile whose epilogue is running (or about to) lies wholly inside the output
     auto group_base = [&](const floatX* buf, int row0, int col0) -> const char* {      // the wave-uniform part of group_ptr
         const size_t off = ((size_t)row0 * g.ldc + col0) * sizeof(floatX);
@@ -503,7 +507,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     auto prefetch_epilogue = [&](int tm0, int tn0, int i) {      // the 32-row block i of this wave's tile
         if (!EPI_READS || i >= TM) return;
         const int wm0 = tm0 + wm * WTM, wn0 = tn0 + wn * WTN;
-        if constexpr (epi_gelu_bwd(EPI)) {
+        if constexpr (epi_reads_aux(EPI)) {
             if (tile_inside) {
 #pragma unroll
                 for (int pass = 0; pass < PASSES; pass++)
@@ -518,11 +522,13 @@ gemm_pipelined_kernel(GemmArgs g) {
                     }
                 return;
             }
+            int eln = lane;       // (PRE_ASM: the lane's row and chunk are formed here, not kept - and spilled - as loop invariants)
+            if constexpr (PRE_ASM) asm volatile("" : "+v"(eln));
 #pragma unroll
             for (int pass = 0; pass < PASSES; pass++)
 #pragma unroll
                 for (int t = 0; t < 4; t++) {
-                    const int row = t * 8 + (lane >> 3), ch = lane & 7;
+                    const int row = t * 8 + (eln >> 3), ch = eln & 7;
                     const int m = wm0 + i * 32 + row;
                     const int n = wn0 + pass * 64 + ch * 8;
                     if (m < g.M && n < g.N) {
@@ -559,7 +565,7 @@ gemm_pipelined_kernel(GemmArgs g) {
     // (bias_ready) half-way through it. As ordinary loads the compiler awaits them with vmcnt(0), which also waits for
     // every hand-issued tile load in flight, so a kernel with such loads cannot request the next tile's first stage
     // before it has claimed its bias (BIAS_LATE below); the product kernels issue and count them by hand (BIAS_ASM).
-    constexpr bool HAS_BIAS = (EPI == EPI_BIAS || epi_gelu_fwd(EPI));
+    constexpr bool HAS_BIAS = (EPI == EPI_BIAS || EPI == EPI_BIAS_RES || epi_gelu_fwd(EPI));
     unsigned biasw[HAS_BIAS ? TN : 1];   // bias of column j*32 + idx of the wave tile in the low 16 bits (lanes 0-31; 0 in lanes 32-63)
     bool bias_lane[HAS_BIAS ? TN : 1];
     // BIAS_ASM: the two bias loads are issued from inline asm and awaited by count, so the next tile's first stage can be
@@ -571,6 +577,9 @@ gemm_pipelined_kernel(GemmArgs g) {
     bool bias_young = false;
     auto request_bias = [&](int n0) {
         if constexpr (HAS_BIAS) {
+            int bln = lane;       // (as above: with epilogue loads in flight a reload of a spilled lane value would wait for them)
+            if constexpr (PRE_ASM) asm volatile("" : "+v"(bln));
+            const int idx = bln & 31, half = bln >> 5;
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 const int n = n0 + wn * WTN + j * 32 + idx;
@@ -587,7 +596,14 @@ gemm_pipelined_kernel(GemmArgs g) {
     };
     auto bias_ready = [&]() {
         if constexpr (HAS_BIAS) {
-            if constexpr (BIAS_ASM) { if (bias_young) wait_vmcnt<CPW>(); else wait_vmcnt<0>(); }
+            if constexpr (BIAS_ASM) {
+                // behind the bias loads: the first block's loads of an epilogue that reads (interior tile: all of them
+                // issued; an edge tile waits for everything) and the late waves' request of the next tile's first stage
+                constexpr int PB = PRE_ASM ? PRE_PB : 0;
+                if (PRE_ASM && !tile_inside) wait_vmcnt<0>();
+                else if (bias_young) wait_vmcnt<PB + CPW>();
+                else wait_vmcnt<PB>();
+            }
 #pragma unroll
             for (int j = 0; j < TN; j++) {
                 asm volatile("" : "+v"(biasw[j]));
@@ -723,11 +739,17 @@ gemm_pipelined_kernel(GemmArgs g) {
                                     }
                                     st_out(auxptr, d.u);
                                     st_out(cptr, y.u);
+                                } else if (EPI == EPI_BIAS_RES) {
+                                    union { u32x4 u; bf16x8 h; } pa;
+                                    pa.u = pre_act[epi_reads_aux(EPI) ? i : 0][epi_reads_aux(EPI) ? pass : 0][t];
+#pragma unroll
+                                    for (int e = 0; e < 8; e++) y.h[e] = (__bf16)((float)x.h[e] + (float)pa.h[e]);
+                                    st_out(cptr, y.u);
                                 } else if (epi_gelu_bwd(EPI)) {
                                     // the product of the rounded gradient and gelu'(pre), as gelu_backward_inplace forms it
                                     // (EPI_DGELU_D: gelu'(pre) is what was stored)
                                     union { u32x4 u; bf16x8 h; } pa;
-                                    pa.u = pre_act[epi_gelu_bwd(EPI) ? i : 0][epi_gelu_bwd(EPI) ? pass : 0][t];
+                                    pa.u = pre_act[epi_reads_aux(EPI) ? i : 0][epi_reads_aux(EPI) ? pass : 0][t];
 #pragma unroll
                                     for (int e = 0; e < 8; e++)
                                         y.h[e] = (__bf16)((EPI == EPI_DGELU_D ? (float)pa.h[e] : gelu_grad_f((float)pa.h[e])) * (float)x.h[e]);
@@ -775,7 +797,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         // values must stay ahead of these loads, nor for split-K partials, whose tiles are long and whose kernel is
         // short of scalar registers).
         constexpr bool EARLY0 = EPI != EPI_ACCUM && !IS_PARTIAL;
-        constexpr bool ROWWISE = LLMK_ROWWISE_LAST && EARLY0 && !TR_ASM && (!epi_gelu_bwd(EPI) || LLMK_ROWWISE_LAST >= 2);
+        constexpr bool ROWWISE = LLMK_ROWWISE_LAST && EARLY0 && !TR_ASM && (!epi_reads_aux(EPI) || LLMK_ROWWISE_LAST >= 2);
         bool early0 = false;
         if (have_next) {
             if constexpr (EARLY0) {

@@ -15,6 +15,12 @@
 #include <vector>
 #include <algorithm>
 
+// 1: the residual adds of the forward pass run as epilogues of the projections that feed them (see the layer loop);
+// 0: the reference's call sequence, projection into a scratch buffer and then the fused residual + LayerNorm kernel
+#ifndef LLMK_FUSE_RESIDUAL
+#define LLMK_FUSE_RESIDUAL 1
+#endif
+
 #include "../../include/llmk.h"
 #include "../../include/llmk_gpt2.h"
 #include "../../include/llmk_data.h"
@@ -464,18 +470,30 @@ void forward_impl(LLMK_GPT2* m, const int* inputs, size_t B, size_t T, bool wait
 
         llmk_matmul_forward(l_qkvr, l_ln1, l_qkvw, l_qkvb, (int)B, (int)T, (int)C, (int)(3 * C), st, nullptr, 1);
         llmk_attention_forward(l_atty, l_att, l_qkvr, (int)B, (int)T, (int)NH, (int)C, st);
-        llmk_matmul_forward(scratch, l_atty, l_attprojw, l_attprojb, (int)B, (int)T, (int)C, (int)C, st, nullptr, 1);
-        llmk_fused_residual_forward5(l_residual2, l_ln2, l_ln2_mean, l_ln2_rstd, residual, scratch, l_ln2w, l_ln2b, (int)(B * T), (int)C, st);
-        llmk_matmul_forward(l_fch_gelu, l_ln2, l_fcw, l_fcb, (int)B, (int)T, (int)C, (int)(4 * C), st, l_fch, gelu_fusion_in_use(m));
-        llmk_matmul_forward(scratch, l_fch_gelu, l_fcprojw, l_fcprojb, (int)B, (int)T, (int)(4 * C), (int)C, st, nullptr, 1);
-        if (l + 1 != L) {
-            xptr n_ln1 = R < 2 ? off(a.ln1, (l + 1) * B * T * C, X) : a.lnf;
-            llmk_fused_residual_forward5(l_residual3, n_ln1, a.ln1_mean + (l + 1) * B * T, a.ln1_rstd + (l + 1) * B * T,
-                                         l_residual2, scratch, off(p.ln1w, (l + 1) * C, X), off(p.ln1b, (l + 1) * C, X),
-                                         (int)(B * T), (int)C, st);
+        // The two projections into the residual stream. The reference runs matmul_forward into a scratch buffer and then
+        // fused_residual_forward5 (train_gpt2.cu:713-727: residual add + LayerNorm); here the add is the projection's
+        // epilogue (llmk_matmul_forward_residual: the same two roundings, the same bits) and a plain LayerNorm follows,
+        // which reads and writes one tensor less per instance.
+        xptr n_ln = l + 1 != L ? (R < 2 ? off(a.ln1, (l + 1) * B * T * C, X) : a.lnf) : a.lnf;
+        float* n_mean = l + 1 != L ? a.ln1_mean + (l + 1) * B * T : a.lnf_mean;
+        float* n_rstd = l + 1 != L ? a.ln1_rstd + (l + 1) * B * T : a.lnf_rstd;
+        xptr n_w = l + 1 != L ? off(p.ln1w, (l + 1) * C, X) : p.lnfw, n_b = l + 1 != L ? off(p.ln1b, (l + 1) * C, X) : p.lnfb;
+        // (Measured on whole steps, both call sequences in one process: 124M -0.80 ms of 58.3, 350M -0.55 ms of 79.0; at 1558M,
+        // whose 1600 columns end in a ragged tile that takes the epilogue's slow path, +0.25 ms of 181.3 - so only for
+        // widths that are whole tiles.)
+        const bool fuse_residual = LLMK_FUSE_RESIDUAL && C % 256 == 0 && X == 2;   // (the fp32 library has no such epilogue)
+        if (fuse_residual) {
+            llmk_matmul_forward_residual(l_residual2, l_atty, l_attprojw, l_attprojb, residual, (int)B, (int)T, (int)C, (int)C, st);
+            llmk_layernorm_forward(l_ln2, l_ln2_mean, l_ln2_rstd, l_residual2, l_ln2w, l_ln2b, (int)B, (int)T, (int)C, st);
+            llmk_matmul_forward(l_fch_gelu, l_ln2, l_fcw, l_fcb, (int)B, (int)T, (int)C, (int)(4 * C), st, l_fch, gelu_fusion_in_use(m));
+            llmk_matmul_forward_residual(l_residual3, l_fch_gelu, l_fcprojw, l_fcprojb, l_residual2, (int)B, (int)T, (int)(4 * C), (int)C, st);
+            llmk_layernorm_forward(n_ln, n_mean, n_rstd, l_residual3, n_w, n_b, (int)B, (int)T, (int)C, st);
         } else {
-            llmk_fused_residual_forward5(l_residual3, a.lnf, a.lnf_mean, a.lnf_rstd, l_residual2, scratch, p.lnfw, p.lnfb,
-                                         (int)(B * T), (int)C, st);
+            llmk_matmul_forward(scratch, l_atty, l_attprojw, l_attprojb, (int)B, (int)T, (int)C, (int)C, st, nullptr, 1);
+            llmk_fused_residual_forward5(l_residual2, l_ln2, l_ln2_mean, l_ln2_rstd, residual, scratch, l_ln2w, l_ln2b, (int)(B * T), (int)C, st);
+            llmk_matmul_forward(l_fch_gelu, l_ln2, l_fcw, l_fcb, (int)B, (int)T, (int)C, (int)(4 * C), st, l_fch, gelu_fusion_in_use(m));
+            llmk_matmul_forward(scratch, l_fch_gelu, l_fcprojw, l_fcprojb, (int)B, (int)T, (int)(4 * C), (int)C, st, nullptr, 1);
+            llmk_fused_residual_forward5(l_residual3, n_ln, n_mean, n_rstd, l_residual2, scratch, n_w, n_b, (int)(B * T), (int)C, st);
         }
     }
     llmk_matmul_forward(a.output, a.lnf, p.wte, nullptr, (int)B, (int)T, (int)C, (int)Vp, st, nullptr, 1);

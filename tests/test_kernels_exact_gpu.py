@@ -92,6 +92,34 @@ def test_forward_projection_is_the_integer_product(C, OC):
     G.check_no_error(L)
 
 
+@pytest.mark.parametrize("M,C,OC", [(N_ROWS, 768, 768), (N_ROWS, 3072, 768), (N_ROWS // 2, 4096, 1024), (N_ROWS // 4, 6400, 1600),
+                                    (N_ROWS // 4 + 72, 768, 832), (640, 768, 768)])
+def test_forward_projection_with_residual_epilogue(M, C, OC):
+    """out = bf16(bf16(x.w^T + b) + residual): the integer product rounded once, then the sum with a residual of
+    non-integers rounded once more - and the same bits as the two kernels it stands for. The projections into the
+    residual stream at the three model widths, a shape with ragged last tiles in both directions, and one too small for
+    the fused epilogue (which then runs the two kernels itself)."""
+    import torch
+    L = G.lib("bf16")
+    x, w, b = ints((M, C), 11), ints((OC, C), 12), ints((OC,), 13, -8, 8)
+    g = torch.Generator(device="cuda"); g.manual_seed(14)
+    res = (torch.randn((M, OC), generator=g, device="cuda") * 3.0).to(torch.bfloat16)
+    out = torch.full((M, OC), 7.0, dtype=torch.bfloat16, device="cuda")
+    for bias in (b, None):
+        L.llmk_matmul_forward_residual(G.ptr(out), G.ptr(x), G.ptr(w), G.ptr(bias) if bias is not None else None, G.ptr(res),
+                                       1, M, C, OC, None)
+        G.sync()
+        proj = exact_nt(x, w) + (bias.float() if bias is not None else 0.0)
+        want = proj.to(torch.bfloat16).float() + res.float()
+        assert_same_bits(out, want, "out = round(round(x.w^T + b) + residual)")
+        two = torch.empty_like(out)
+        L.llmk_matmul_forward(G.ptr(two), G.ptr(x), G.ptr(w), G.ptr(bias) if bias is not None else None, 1, M, C, OC, None, None, 1)
+        L.llmk_residual_forward(G.ptr(two), G.ptr(res), G.ptr(two), M * OC, None)
+        G.sync()
+        assert torch.equal(out, two), "the fused epilogue and the two kernels differ"
+    G.check_no_error(L)
+
+
 @pytest.mark.parametrize("C,OC", [(768, 3072), (1024, 4096), (1600, 6400)])
 def test_forward_projection_with_gelu_epilogue(C, OC):
     """The fc layer with GELU in the GEMM's epilogue: the pre-activation output is the exact product (operands scaled by
