@@ -118,6 +118,11 @@ def run_cases(L, reps=20, only=(), emit=print, others=()):
             out_t = torch.empty(N, OC, device=dev, dtype=torch.bfloat16)
             report(f"matmul_forward {nm} K={K} OC={OC}",
                    measure(lambda: L.llmk_matmul_forward(p(out_t), p(inp), p(w), p(bias), B, T, K, OC, None, None, 0)))
+            if nm in ("attproj", "fcproj"):                     # the projections into the residual stream, with the add as their epilogue
+                res = randn(N, OC)
+                report(f"matmul_forward+residual {nm} K={K} OC={OC}",
+                       measure(lambda: L.llmk_matmul_forward_residual(p(out_t), p(inp), p(w), p(bias), p(res), B, T, K, OC, None)))
+                del res
             if nm == "fc":
                 pre = torch.empty_like(out_t)
                 report(f"matmul_forward+gelu {nm} K={K} OC={OC}",
