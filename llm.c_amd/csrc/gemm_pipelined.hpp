@@ -487,7 +487,9 @@ gemm_pipelined_kernel(GemmArgs g) {
     // of little else; 1-2 % slower for the forward epilogues with activation math. The two backward GELU epilogues take
     // this form: it is also what their hand-issued loads below address by)
     constexpr bool UNIFORM_GROUPS = epi_reads_aux(EPI);
-    bool tile_inside = false;            // the tile whose epilogue is running (or about to) lies wholly inside the output
+    // the wave's part of the tile whose epilogue is running (or about to) lies wholly inside the output: all rows of the tile
+    // and the wave's own WTN columns (a tile on the ragged right edge still has waves like that when N is a multiple of WTN)
+    bool tile_inside = false;
     auto group_base = [&](const floatX* buf, int row0, int col0) -> const char* {      // the wave-uniform part of group_ptr
         const size_t off = ((size_t)row0 * g.ldc + col0) * sizeof(floatX);
         const unsigned lo = (unsigned)__builtin_amdgcn_readfirstlane((int)(unsigned)off);
@@ -868,7 +870,7 @@ gemm_pipelined_kernel(GemmArgs g) {
             // change sit there, two blocks of output stores ahead of the next tile's second stage and two behind it.
             const unsigned cur = buf_of(nst - 1);
             request_bias(n0);
-            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
+            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + wn * WTN + WTN <= g.N;
             prefetch_epilogue(m0, n0, 0);
             prefetch_epilogue(m0, n0, 1);
             bf16x8 fbs[3][TN], far[2][3];
@@ -924,7 +926,7 @@ gemm_pipelined_kernel(GemmArgs g) {
         } else {
             const unsigned cur = buf_of(nst - 1);
             request_bias(n0);                                     // nothing of this wave is in flight here (kernels with a bias)
-            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + BN <= g.N;
+            tile_inside = UNIFORM_GROUPS && m0 + BM <= g.M && n0 + wn * WTN + WTN <= g.N;
             prefetch_epilogue(m0, n0, 0);
             read_frags(cur, S1{}, fa1, fb1);
             await_frags(fa0, fb0, Younger{});

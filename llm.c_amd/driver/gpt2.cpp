@@ -478,10 +478,10 @@ void forward_impl(LLMK_GPT2* m, const int* inputs, size_t B, size_t T, bool wait
         float* n_mean = l + 1 != L ? a.ln1_mean + (l + 1) * B * T : a.lnf_mean;
         float* n_rstd = l + 1 != L ? a.ln1_rstd + (l + 1) * B * T : a.lnf_rstd;
         xptr n_w = l + 1 != L ? off(p.ln1w, (l + 1) * C, X) : p.lnfw, n_b = l + 1 != L ? off(p.ln1b, (l + 1) * C, X) : p.lnfb;
-        // (Measured on whole steps, both call sequences in one process: 124M -0.80 ms of 58.3, 350M -0.55 ms of 79.0; at 1558M,
-        // whose 1600 columns end in a ragged tile that takes the epilogue's slow path, +0.25 ms of 181.3 - so only for
-        // widths that are whole tiles.)
-        const bool fuse_residual = LLMK_FUSE_RESIDUAL && C % 256 == 0 && X == 2;   // (the fp32 library has no such epilogue)
+        // (Measured on whole steps, both call sequences in one process: 124M -0.80 ms of 58.3, 350M -0.55 ms of 79.0, 1558M
+        // -0.9 ms of 183.9. Widths that are multiples of 64: a wave's 64 columns are then all inside the output or all
+        // outside, which is what the epilogue's counted loads need on the ragged last tile column of the 1600-wide model.)
+        const bool fuse_residual = LLMK_FUSE_RESIDUAL && C % 64 == 0 && X == 2;   // (the fp32 library has no such epilogue)
         if (fuse_residual) {
             llmk_matmul_forward_residual(l_residual2, l_atty, l_attprojw, l_attprojb, residual, (int)B, (int)T, (int)C, (int)C, st);
             llmk_layernorm_forward(l_ln2, l_ln2_mean, l_ln2_rstd, l_residual2, l_ln2w, l_ln2b, (int)B, (int)T, (int)C, st);
